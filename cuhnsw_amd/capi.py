@@ -1,0 +1,137 @@
+"""ctypes binding of the C ABI (include/cuhnsw_amd.h) — the same entry points the
+pybind11 module wraps, reachable without pybind11 (foreign-function callers, the
+benchmark's device-pointer search)."""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcuhnsw_amd.so")
+
+SYMBOLS = [
+    "cuhnsw_create", "cuhnsw_destroy", "cuhnsw_last_error", "cuhnsw_init",
+    "cuhnsw_set_data", "cuhnsw_set_random_levels", "cuhnsw_build_graph",
+    "cuhnsw_save_index", "cuhnsw_load_index", "cuhnsw_search_knn",
+    "cuhnsw_search_knn_device", "cuhnsw_num_data", "cuhnsw_num_dims",
+    "cuhnsw_max_level", "cuhnsw_enter_point", "cuhnsw_has_device",
+    "cuhnsw_last_build_seconds", "cuhnsw_set_tunable",
+]
+
+_lib = None
+
+
+def load():
+  """Loads libcuhnsw_amd.so; raises OSError if it has not been built."""
+  global _lib
+  if _lib is not None:
+    return _lib
+  if not os.path.exists(LIB_PATH):
+    raise OSError("libcuhnsw_amd.so is not built; run `python -m cuhnsw_amd.build`")
+  l = ctypes.CDLL(LIB_PATH)
+  vp, ci, cd = ctypes.c_void_p, ctypes.c_int, ctypes.c_double
+  l.cuhnsw_create.argtypes = [ctypes.POINTER(vp)]
+  l.cuhnsw_destroy.argtypes = [vp]
+  l.cuhnsw_destroy.restype = None
+  l.cuhnsw_last_error.argtypes = [vp]
+  l.cuhnsw_last_error.restype = ctypes.c_char_p
+  l.cuhnsw_init.argtypes = [vp, ctypes.c_char_p]
+  l.cuhnsw_set_data.argtypes = [vp, vp, ci, ci]
+  l.cuhnsw_set_random_levels.argtypes = [vp, vp, ci]
+  l.cuhnsw_build_graph.argtypes = [vp]
+  l.cuhnsw_save_index.argtypes = [vp, ctypes.c_char_p]
+  l.cuhnsw_load_index.argtypes = [vp, ctypes.c_char_p]
+  l.cuhnsw_search_knn.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp]
+  l.cuhnsw_search_knn_device.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp, vp, ctypes.POINTER(ctypes.c_float)]
+  for name in ("cuhnsw_num_data", "cuhnsw_num_dims", "cuhnsw_max_level", "cuhnsw_enter_point"):
+    getattr(l, name).argtypes = [vp]
+  l.cuhnsw_has_device.argtypes = []
+  l.cuhnsw_last_build_seconds.argtypes = [vp]
+  l.cuhnsw_last_build_seconds.restype = cd
+  l.cuhnsw_set_tunable.argtypes = [vp, ctypes.c_char_p, cd]
+  _lib = l
+  return l
+
+
+def has_device():
+  return bool(load().cuhnsw_has_device())
+
+
+class Engine:
+  """One engine handle; methods map 1:1 onto the C entry points and raise
+  RuntimeError with the engine's message on failure."""
+
+  def __init__(self):
+    self._l = load()
+    self._h = ctypes.c_void_p()
+    if self._l.cuhnsw_create(ctypes.byref(self._h)) != 0:
+      raise RuntimeError("cuhnsw_create failed: " + self._l.cuhnsw_last_error(None).decode())
+
+  def close(self):
+    if self._h:
+      self._l.cuhnsw_destroy(self._h)
+      self._h = ctypes.c_void_p()
+
+  def __del__(self):
+    try:
+      self.close()
+    except Exception:  # pylint: disable=broad-except
+      pass
+
+  def _check(self, rc):
+    if rc != 0:
+      raise RuntimeError(self._l.cuhnsw_last_error(self._h).decode())
+
+  def init(self, opt_path):
+    """0 ok, 1 unreadable option file, 2 invalid dist_type (no exception, like the C call)."""
+    return self._l.cuhnsw_init(self._h, os.fsencode(opt_path))
+
+  def set_data(self, data):
+    data = np.ascontiguousarray(data, dtype=np.float32)
+    if data.ndim != 2:
+      raise RuntimeError("data must be 2d array")
+    self._check(self._l.cuhnsw_set_data(self._h, data.ctypes.data, data.shape[0], data.shape[1]))
+
+  def set_random_levels(self, levels):
+    levels = np.ascontiguousarray(levels, dtype=np.int32)
+    self._check(self._l.cuhnsw_set_random_levels(self._h, levels.ctypes.data, levels.shape[0]))
+
+  def build_graph(self):
+    self._check(self._l.cuhnsw_build_graph(self._h))
+
+  def save_index(self, path):
+    self._check(self._l.cuhnsw_save_index(self._h, os.fsencode(path)))
+
+  def load_index(self, path):
+    self._check(self._l.cuhnsw_load_index(self._h, os.fsencode(path)))
+
+  def search_knn(self, queries, topk, ef_search):
+    queries = np.ascontiguousarray(queries, dtype=np.float32)
+    if queries.ndim == 1:
+      queries = queries[None, :]
+    if queries.shape[1] != self.num_dims:
+      raise RuntimeError("query dimension differs from the index dimension")
+    nq = queries.shape[0]
+    nns = np.empty((nq, topk), dtype=np.int32)
+    dists = np.empty((nq, topk), dtype=np.float32)
+    found = np.empty(nq, dtype=np.int32)
+    self._check(self._l.cuhnsw_search_knn(self._h, queries.ctypes.data, nq, topk, ef_search,
+                                          nns.ctypes.data, dists.ctypes.data, found.ctypes.data))
+    return nns, dists, found
+
+  def search_knn_device(self, q_ptr, nq, topk, ef_search, nns_ptr, dist_ptr, found_ptr, stats_ptr=None):
+    """All pointers are device addresses (ints).  Returns the kernel time in ms."""
+    ms = ctypes.c_float(0.0)
+    self._check(self._l.cuhnsw_search_knn_device(self._h, q_ptr, nq, topk, ef_search, nns_ptr, dist_ptr,
+                                                 found_ptr, stats_ptr, ctypes.byref(ms)))
+    return ms.value
+
+  def set_tunable(self, name, value):
+    if self._l.cuhnsw_set_tunable(self._h, name.encode(), float(value)) != 0:
+      raise RuntimeError("unknown tunable " + name)
+
+  num_data = property(lambda s: s._l.cuhnsw_num_data(s._h))
+  num_dims = property(lambda s: s._l.cuhnsw_num_dims(s._h))
+  max_level = property(lambda s: s._l.cuhnsw_max_level(s._h))
+  enter_point = property(lambda s: s._l.cuhnsw_enter_point(s._h))
+  last_build_seconds = property(lambda s: s._l.cuhnsw_last_build_seconds(s._h))

@@ -1,0 +1,413 @@
+// Wavefront-level building blocks shared by the search and build kernels (gfx950,
+// 64-lane wavefronts, one wavefront per query / inserted node).
+//
+//   * distances: a 64-lane wavefront works on FOUR rows at a time, 16 lanes per row,
+//     each lane loading float4 (dwordx4) chunks of the row, so one load instruction
+//     of the wavefront fetches 4 x 256 contiguous bytes.  The 16 lanes are reduced
+//     with DPP (quad_perm, row_half_mirror, row_mirror); no LDS, no barrier.
+//     Replaces dot / squaresum / GetDistanceByVec of the reference
+//     (cpp/include/cuda_dist_kernels.cuh:13-124), which reduce over a 32-thread
+//     block through shared memory.
+//   * candidate queues live in LDS and reproduce libstdc++ heaps (heap_emul.h);
+//     replaces the global-memory, thread-0 heap of the reference
+//     (cpp/include/cuda_heap_kernels.cuh:13-49) and its GetCand / CheckAlreadyExists
+//     scans (cpp/include/cuda_utils_kernels.cuh:50-151).
+//   * the visited set is an exact bitmap per resident wavefront (one bit per node,
+//     global memory, cleared through an undo list), not the lossy direct-mapped
+//     table of the reference (cpp/include/cuda_utils_kernels.cuh:185-210).
+//
+// Canonical fp32 distance arithmetic: element i is accumulated with one fused
+// multiply-add into partial sum (i mod 64) in increasing i; the 64 partials are
+// combined by a pairwise adjacent tree (s = 1,2 inside a lane, s = 4..32 across the
+// 16 lanes).  The key used for ordering is 1 - dot (hnswlib) or the squared L2.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "heap_emul.h"
+#include "index_file.h"
+#include "options.h"
+
+namespace cuhnsw_amd {
+
+struct DevIndex {
+  const float* vectors;      // N x Dp, rows zero padded to Dp (multiple of 32 floats)
+  const uint64_t* labels;    // N, or null when labels are the internal ids
+  uint32_t* links0;          // N x S0
+  uint32_t* linksU;          // upper rows x SU
+  const int64_t* upper_off;  // N
+  const int* levels;         // N
+  float* dists0;             // build only: key of every level-0 link
+  float* distsU;             // build only
+  int N, D, Dp, S0, SU, max_m, max_m0, maxlevel;
+  uint32_t enterpoint;
+};
+
+// per resident wavefront scratch: LDS pointers + this wavefront's global slot
+struct Scratch {
+  HeapEnt* top;        // LDS, ef + 1 entries
+  HeapEnt* cand;       // LDS, cand_lds entries
+  HeapEnt* cand_glob;  // global overflow of the candidate queue
+  int cand_lds, cand_glob_cap;
+  uint32_t* nbuf;      // LDS, lcap ids
+  float* dbuf;         // LDS, lcap keys
+  float4* qlds;        // LDS copy of the query (only when the query is not kept in registers)
+  uint32_t* bitmap;    // global, one bit per node
+  uint32_t* undo;      // global, ids whose bit is set
+  int undo_cap;
+  int bitmap_words;
+};
+
+struct SearchState {
+  int top_size, cand_size;
+  float lower;
+  int undo_cnt;
+  int n_dist, n_hops, n_dist_upper, n_sweeps;
+  int fail;
+};
+
+struct LdsHeap {
+  HeapEnt* a;
+  __device__ __forceinline__ HeapEnt get(int i) const { return a[i]; }
+  __device__ __forceinline__ void set(int i, HeapEnt e) { a[i] = e; }
+};
+struct SplitHeap {
+  HeapEnt* lds;
+  HeapEnt* glob;
+  int nlds;
+  __device__ __forceinline__ HeapEnt get(int i) const { return i < nlds ? lds[i] : glob[i - nlds]; }
+  __device__ __forceinline__ void set(int i, HeapEnt e) {
+    if (i < nlds) lds[i] = e; else glob[i - nlds] = e;
+  }
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+// sum over each group of 16 consecutive lanes; every lane of the group gets the same bits.
+// Must be executed with all 64 lanes active.
+__device__ __forceinline__ float reduce16(float x) {
+  x = x + dpp_move<0xB1>(x);   // quad_perm [1,0,3,2]
+  x = x + dpp_move<0x4E>(x);   // quad_perm [2,3,0,1]
+  x = x + dpp_move<0x141>(x);  // row_half_mirror
+  x = x + dpp_move<0x140>(x);  // row_mirror
+  return x;
+}
+__device__ __forceinline__ float wave_min(float x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x = fminf(x, __shfl_xor(x, m, 64));
+  return x;
+}
+
+template <int DT>
+__device__ __forceinline__ void acc4(const float4 q, const float4 v, float& ax, float& ay, float& az, float& aw) {
+  if (DT == DIST_DOT) {
+    ax = __builtin_fmaf(q.x, v.x, ax);
+    ay = __builtin_fmaf(q.y, v.y, ay);
+    az = __builtin_fmaf(q.z, v.z, az);
+    aw = __builtin_fmaf(q.w, v.w, aw);
+  } else {
+    float tx = q.x - v.x, ty = q.y - v.y, tz = q.z - v.z, tw = q.w - v.w;
+    ax = __builtin_fmaf(tx, tx, ax);
+    ay = __builtin_fmaf(ty, ty, ay);
+    az = __builtin_fmaf(tz, tz, az);
+    aw = __builtin_fmaf(tw, tw, aw);
+  }
+}
+// RAW = false: ordering key (1 - dot | squared L2); RAW = true: API value (-dot | squared L2)
+template <int DT, bool RAW>
+__device__ __forceinline__ float finish16(float ax, float ay, float az, float aw) {
+  float s = (ax + ay) + (az + aw);
+  s = reduce16(s);
+  if (DT == DIST_DOT) return RAW ? -s : 1.0f - s;
+  return s;
+}
+
+// Query kept in registers: lane `sub` of each 16-lane group holds float4 chunks
+// sub, sub+16, ... (QR of them).  QR == 0 selects the LDS copy instead.
+template <int QR>
+struct QVec {
+  float4 q[QR > 0 ? QR : 1];
+};
+
+// fills the query holder from a row of D floats (any alignment)
+template <int QR>
+__device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const float* src, int D, int Dp, int lane) {
+  if (QR > 0) {
+    const int sub = lane & 15;
+#pragma unroll
+    for (int k = 0; k < (QR > 0 ? QR : 1); ++k) {
+      int i = 4 * (sub + 16 * k);
+      float4 t;
+      t.x = i + 0 < D ? src[i + 0] : 0.0f;
+      t.y = i + 1 < D ? src[i + 1] : 0.0f;
+      t.z = i + 2 < D ? src[i + 2] : 0.0f;
+      t.w = i + 3 < D ? src[i + 3] : 0.0f;
+      qv.q[k] = t;
+    }
+  } else {
+    const int chunks = ((Dp >> 2) + 15) / 16 * 16;
+    for (int c = lane; c < chunks; c += 64) {
+      int i = 4 * c;
+      float4 t;
+      t.x = i + 0 < D ? src[i + 0] : 0.0f;
+      t.y = i + 1 < D ? src[i + 1] : 0.0f;
+      t.z = i + 2 < D ? src[i + 2] : 0.0f;
+      t.w = i + 3 < D ? src[i + 3] : 0.0f;
+      qlds[c] = t;
+    }
+    __syncthreads();
+  }
+}
+
+// keys of ids[0..n) (LDS) against the query -> out[0..n) (LDS).  n is wavefront-uniform.
+template <int DT, int QR, bool RAW>
+__device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds,
+                                          const uint32_t* ids, int n, float* out, int lane) {
+  const int g = lane >> 4, sub = lane & 15;
+  const int rowlen = ix.Dp >> 2;
+  const float4* rows = reinterpret_cast<const float4*>(ix.vectors);
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (QR > 0) {
+    constexpr int R = QR > 0 ? QR : 1;
+    constexpr int U = R == 1 ? 4 : (R == 2 ? 2 : 1);  // groups of 4 rows in flight
+    for (int r = 0; r < n; r += 4 * U) {
+      float4 v[U][R];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        int idx = r + 4 * u + g;
+        uint32_t id = ids[idx < n ? idx : n - 1];
+        const float4* p = rows + (size_t)id * rowlen + sub;
+#pragma unroll
+        for (int k = 0; k < R; ++k) v[u][k] = (sub + 16 * k < rowlen) ? p[16 * k] : zero;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
+#pragma unroll
+        for (int k = 0; k < R; ++k) acc4<DT>(qv.q[k], v[u][k], ax, ay, az, aw);
+        float key = finish16<DT, RAW>(ax, ay, az, aw);
+        int idx = r + 4 * u + g;
+        if (sub == 0 && idx < n) out[idx] = key;
+      }
+    }
+  } else {
+    const int nk = (rowlen + 15) >> 4;
+    for (int r = 0; r < n; r += 4) {
+      int idx = r + g;
+      uint32_t id = ids[idx < n ? idx : n - 1];
+      const float4* p = rows + (size_t)id * rowlen + sub;
+      float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
+#pragma unroll 4
+      for (int k = 0; k < nk; ++k) {
+        float4 v = (sub + 16 * k < rowlen) ? p[16 * k] : zero;
+        acc4<DT>(qlds[sub + 16 * k], v, ax, ay, az, aw);
+      }
+      float key = finish16<DT, RAW>(ax, ay, az, aw);
+      if (sub == 0 && idx < n) out[idx] = key;
+    }
+  }
+}
+
+__device__ __forceinline__ const uint32_t* link_row(const DevIndex& ix, uint32_t node, int level) {
+  return level == 0 ? ix.links0 + (size_t)node * ix.S0 : ix.linksU + (size_t)(ix.upper_off[node] + level - 1) * ix.SU;
+}
+__device__ __forceinline__ int row_stride(const DevIndex& ix, int level) { return level == 0 ? ix.S0 : ix.SU; }
+
+// marks one id visited (lane 0 does it); returns nothing, logs it for the undo
+__device__ __forceinline__ void visit_single(Scratch& s, SearchState& st, uint32_t id, int lane) {
+  if (lane == 0) {
+    atomicOr(&s.bitmap[id >> 5], 1u << (id & 31));
+    if (st.undo_cnt < s.undo_cap) s.undo[st.undo_cnt] = id;
+  }
+  st.undo_cnt += 1;
+}
+
+// Reads a link row, marks its ids visited and compacts the ones seen for the first
+// time into s.nbuf (stored order kept).  Returns how many.
+__device__ __forceinline__ int visit_row(const uint32_t* row, int S, Scratch& s, SearchState& st, int lane) {
+  int n = 0;
+  for (int base = 0; base < S; base += 64) {
+    uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
+    bool newly = false;
+    if (id != kEmpty) {
+      uint32_t bit = 1u << (id & 31);
+      uint32_t old = atomicOr(&s.bitmap[id >> 5], bit);
+      newly = (old & bit) == 0;
+    }
+    unsigned long long mask = __ballot(newly);
+    int pos = n + __popcll(mask & ((1ull << lane) - 1ull));
+    if (newly) {
+      s.nbuf[pos] = id;
+      int u = st.undo_cnt + pos;
+      if (u < s.undo_cap) s.undo[u] = id;
+    }
+    n += __popcll(mask);
+  }
+  st.undo_cnt += n;
+  return n;
+}
+
+// Reads a link row and compacts its valid ids into s.nbuf without touching the visited set.
+__device__ __forceinline__ int load_row(const uint32_t* row, int S, Scratch& s, int lane) {
+  int n = 0;
+  for (int base = 0; base < S; base += 64) {
+    uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
+    bool valid = id != kEmpty;
+    unsigned long long mask = __ballot(valid);
+    int pos = n + __popcll(mask & ((1ull << lane) - 1ull));
+    if (valid) s.nbuf[pos] = id;
+    n += __popcll(mask);
+  }
+  return n;
+}
+
+// clears the bits this wavefront set; leaves the slot's bitmap all zero
+__device__ __forceinline__ void undo_visited(Scratch& s, SearchState& st, int lane) {
+  if (st.undo_cnt <= s.undo_cap) {
+    for (int i = lane; i < st.undo_cnt; i += 64) s.bitmap[s.undo[i] >> 5] = 0u;
+  } else {
+    for (int w = lane; w < s.bitmap_words; w += 64) s.bitmap[w] = 0u;
+  }
+  __threadfence();
+  st.undo_cnt = 0;
+}
+
+// Offers nbuf/dbuf[0..n) to the two queues in stored order (hnswlib's accept rule,
+// identical to the reference's, cpp/include/cuda_utils_kernels.cuh:220-225).
+// Executed by ONE lane.
+__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, int n, int ef) {
+  LdsHeap top{s.top};
+  SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
+  const int cand_cap = s.cand_lds + s.cand_glob_cap;
+  for (int t = 0; t < n; ++t) {
+    float d = s.dbuf[t];
+    if (st.top_size < ef || st.lower > d) {
+      if (st.cand_size >= cand_cap) {
+        st.fail = 1;
+        return;
+      }
+      HeapEnt e;
+      e.key = d;
+      e.id = s.nbuf[t];
+      heap_push<true>(cand, st.cand_size, e);
+      heap_push<false>(top, st.top_size, e);
+      if (st.top_size > ef) heap_pop<false>(top, st.top_size);
+      st.lower = s.top[0].key;
+    }
+  }
+}
+
+// Best-first search of one level (hnswlib searchBaseLayerST / searchBaseLayer).
+// On entry s.nbuf[0..n_seed) holds seed ids that are already marked visited; on
+// exit s.top[0..st.top_size) is the result max-heap.  BUILD selects hnswlib's
+// construction-time stop rule.
+template <int DT, int QR, bool BUILD>
+__device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
+                                             SearchState& st, int n_seed, int lane) {
+  SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
+  const int S = row_stride(ix, level);
+  int n = n_seed;
+  while (true) {
+    if (n > 0) {
+      dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      st.n_dist += n;
+    }
+    __syncthreads();
+    int cid = -1;
+    if (lane == 0) {
+      accept_list(s, st, n, ef);
+      if (!st.fail && st.cand_size > 0) {
+        HeapEnt c = cand.get(0);
+        bool stop = BUILD ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
+        if (!stop) {
+          cid = (int)c.id;
+          heap_pop<true>(cand, st.cand_size);
+        }
+      }
+    }
+    cid = __builtin_amdgcn_readfirstlane(cid);
+    __syncthreads();
+    if (cid < 0) break;
+    st.n_hops += 1;
+    n = visit_row(link_row(ix, (uint32_t)cid, level), S, s, st, lane);
+    __syncthreads();
+  }
+  st.top_size = __builtin_amdgcn_readfirstlane(st.top_size);
+  st.cand_size = __builtin_amdgcn_readfirstlane(st.cand_size);
+  st.fail = __builtin_amdgcn_readfirstlane(st.fail);
+}
+
+// Greedy descent through levels from_level .. to_level+1 (hnswlib searchKnn upper
+// loop; cpp/include/cuda_search_kernels.cuh:22-66 in the reference): each sweep
+// scans the neighbour list captured at its start and moves to the strictly
+// closest entry, which for a strict running minimum is the first occurrence of the
+// list minimum.
+template <int DT, int QR>
+__device__ __forceinline__ void descend(const DevIndex& ix, const QVec<QR>& qv, int from_level, int to_level,
+                                        uint32_t& cur, float& dcur, Scratch& s, SearchState& st, int lane) {
+  for (int level = from_level; level > to_level; --level) {
+    bool changed = true;
+    while (changed) {
+      changed = false;
+      int n = load_row(link_row(ix, cur, level), ix.SU, s, lane);
+      __syncthreads();
+      st.n_sweeps += 1;
+      if (n == 0) break;
+      dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      st.n_dist_upper += n;
+      __syncthreads();
+      float best = INFINITY;
+      int bidx = -1;
+      for (int base = 0; base < n; base += 64) {
+        int t = base + lane;
+        float d = t < n ? s.dbuf[t] : INFINITY;
+        float m = wave_min(d);
+        if (m < best) {
+          best = m;
+          unsigned long long mask = __ballot(d == m);
+          bidx = base + __ffsll((long long)mask) - 1;
+        }
+      }
+      if (bidx >= 0 && best < dcur) {
+        dcur = best;
+        cur = s.nbuf[bidx];
+        changed = true;
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// key of one node against the query (all lanes return it)
+template <int DT, int QR>
+__device__ __forceinline__ float dist_single(const DevIndex& ix, const QVec<QR>& qv, uint32_t id, Scratch& s, int lane) {
+  if (lane == 0) s.nbuf[0] = id;
+  __syncthreads();
+  dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, 1, s.dbuf, lane);
+  __syncthreads();
+  float d = s.dbuf[0];
+  __syncthreads();
+  return d;
+}
+
+// Ascending (key, tie) ranking of n LDS entries into out_id / out_key (rank sort,
+// O(n^2 / 64) per lane).  tie[] may be null (then the id breaks ties).
+__device__ __forceinline__ void rank_sort(const HeapEnt* in, const uint64_t* tie, int n, uint32_t* out_id, float* out_key,
+                                          int lane) {
+  for (int e = lane; e < n; e += 64) {
+    HeapEnt me = in[e];
+    uint64_t mt = tie ? tie[e] : (uint64_t)me.id;
+    int rank = 0;
+    for (int f = 0; f < n; ++f) {
+      HeapEnt o = in[f];
+      uint64_t ot = tie ? tie[f] : (uint64_t)o.id;
+      rank += (o.key < me.key || (o.key == me.key && ot < mt)) ? 1 : 0;
+    }
+    out_id[rank] = me.id;
+    out_key[rank] = me.key;
+  }
+}
+
+}  // namespace cuhnsw_amd

@@ -1,0 +1,584 @@
+// Host engine and C ABI of libcuhnsw_amd.so.
+//
+// Counterpart of the reference's host class cuhnsw::CuHNSW
+// (cpp/include/cuhnsw.hpp:61-112, cpp/src/cuhnsw_base.cu, cpp/src/cuhnsw_build.cu).
+// Differences by design: the whole multi-level index stays resident in HBM in flat
+// fixed-stride rows (the reference re-flattens and re-uploads the graph on every
+// search call, cpp/src/cuhnsw_build.cu:226-253, and once per upper level for the
+// descent, :25-94); there is no per-level host graph container; HIP runtime calls
+// are made directly (no Thrust).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/cuhnsw_amd.h"
+#include "index_file.h"
+#include "kernels.h"
+#include "options.h"
+
+namespace cuhnsw_amd {
+
+#define HIP_CHECK(expr)                                                                              \
+  do {                                                                                               \
+    hipError_t err_ = (expr);                                                                        \
+    if (err_ != hipSuccess)                                                                          \
+      throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(err_) + " at " #expr); \
+  } while (0)
+
+static bool device_present() {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return n > 0;
+}
+
+template <typename T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+  }
+  // grows (never shrinks); contents are not preserved
+  void reserve(size_t want) {
+    if (want <= n) return;
+    release();
+    HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&p), want * sizeof(T)));
+    n = want;
+  }
+  ~DevBuf() { release(); }
+};
+
+class Engine {
+ public:
+  Options opt;
+  int dist_type = DIST_DOT;
+  HostIndex host;
+  bool have_data = false, have_levels = false, have_graph = false;
+  bool host_links_stale = false;  // device links are newer than host.links0 / linksU
+  bool has_device = false;
+  int num_cus = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  std::string err;
+  double last_build_seconds = 0.0;
+
+  // tunables
+  int build_batch = 16384;
+  int search_slots = 0;
+  int cand_lds_override = 0;
+  int hnswlib_dist = 0;
+
+  // resident index
+  int Dp = 0;
+  DevBuf<float> d_vectors;
+  DevBuf<uint64_t> d_labels;
+  DevBuf<uint32_t> d_links0, d_linksU;
+  DevBuf<int64_t> d_upper_off;
+  DevBuf<int> d_levels;
+  // per-wavefront slots
+  DevBuf<uint32_t> d_bitmaps, d_undo;
+  DevBuf<HeapEnt> d_cand_glob;
+  SlotPool pool{};
+  int pool_slots = 0;
+  DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count
+  // staging for the host-pointer search entry point
+  DevBuf<float> d_q, d_dist;
+  DevBuf<int> d_nns, d_found;
+
+  Engine() {
+    has_device = device_present();
+    if (has_device) {
+      hipDeviceProp_t prop;
+      HIP_CHECK(hipGetDeviceProperties(&prop, 0));
+      num_cus = prop.multiProcessorCount;
+      HIP_CHECK(hipStreamCreate(&stream));
+      HIP_CHECK(hipEventCreate(&ev0));
+      HIP_CHECK(hipEventCreate(&ev1));
+      d_ctl.reserve(4);
+    }
+  }
+  ~Engine() {
+    if (ev0) (void)hipEventDestroy(ev0);
+    if (ev1) (void)hipEventDestroy(ev1);
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+
+  void need_device() const {
+    if (!has_device) throw std::runtime_error("no HIP device available: this call needs a GPU");
+  }
+
+  static int padded_dims(int D) { return (D + 31) / 32 * 32; }
+  int qr() const {
+    int chunks16 = ((Dp >> 2) + 15) / 16;
+    if (chunks16 <= 1) return 1;
+    if (chunks16 <= 2) return 2;
+    if (chunks16 <= 4) return 4;
+    return 0;
+  }
+
+  DevIndex dev_index(float* dists0 = nullptr, float* distsU = nullptr) const {
+    DevIndex ix;
+    ix.vectors = d_vectors.p;
+    ix.labels = host.labelled ? d_labels.p : nullptr;
+    ix.links0 = d_links0.p;
+    ix.linksU = d_linksU.p;
+    ix.upper_off = d_upper_off.p;
+    ix.levels = d_levels.p;
+    ix.dists0 = dists0;
+    ix.distsU = distsU;
+    ix.N = host.N; ix.D = host.D; ix.Dp = Dp; ix.S0 = host.S0; ix.SU = host.SU;
+    ix.max_m = host.max_m; ix.max_m0 = host.max_m0; ix.maxlevel = host.maxlevel;
+    ix.enterpoint = host.enterpoint;
+    return ix;
+  }
+
+  // ---- option / data / level plumbing -------------------------------------------------
+  int init(const char* path) {
+    Options o;
+    int dt = DIST_DOT;
+    int rc = load_options(path ? path : "", o, dt);
+    if (rc == 0) {
+      opt = o;
+      dist_type = dt;
+    }
+    return rc;
+  }
+
+  void upload_vectors() {
+    Dp = padded_dims(host.D);
+    d_vectors.reserve((size_t)host.N * Dp);
+    HIP_CHECK(hipMemsetAsync(d_vectors.p, 0, (size_t)host.N * Dp * sizeof(float), stream));
+    HIP_CHECK(hipMemcpy2DAsync(d_vectors.p, (size_t)Dp * 4, host.vectors.data(), (size_t)host.D * 4, (size_t)host.D * 4,
+                               (size_t)host.N, hipMemcpyHostToDevice, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+  }
+
+  void set_data(const float* data, int n, int d) {
+    if (!data || n <= 0 || d <= 0) throw std::runtime_error("set_data: empty data");
+    need_device();
+    host = HostIndex();
+    host.N = n;
+    host.D = d;
+    host.vectors.assign(data, data + (size_t)n * d);
+    have_levels = have_graph = host_links_stale = false;
+    upload_vectors();
+    have_data = true;
+  }
+
+  void upload_structure() {
+    d_levels.reserve((size_t)host.N);
+    d_upper_off.reserve((size_t)host.N);
+    d_links0.reserve((size_t)host.N * host.S0);
+    d_linksU.reserve(std::max<size_t>((size_t)host.upper_rows * host.SU, 1));
+    HIP_CHECK(hipMemcpyAsync(d_levels.p, host.levels.data(), (size_t)host.N * 4, hipMemcpyHostToDevice, stream));
+    HIP_CHECK(hipMemcpyAsync(d_upper_off.p, host.upper_off.data(), (size_t)host.N * 8, hipMemcpyHostToDevice, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+  }
+  void upload_links() {
+    HIP_CHECK(hipMemcpyAsync(d_links0.p, host.links0.data(), host.links0.size() * 4, hipMemcpyHostToDevice, stream));
+    if (!host.linksU.empty())
+      HIP_CHECK(hipMemcpyAsync(d_linksU.p, host.linksU.data(), host.linksU.size() * 4, hipMemcpyHostToDevice, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+  }
+  void download_links() {
+    HIP_CHECK(hipMemcpyAsync(host.links0.data(), d_links0.p, host.links0.size() * 4, hipMemcpyDeviceToHost, stream));
+    if (!host.linksU.empty())
+      HIP_CHECK(hipMemcpyAsync(host.linksU.data(), d_linksU.p, host.linksU.size() * 4, hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+    host_links_stale = false;
+  }
+
+  void set_random_levels(const int* levels, int n) {
+    if (!have_data) throw std::runtime_error("set_random_levels: call set_data first");
+    if (n != host.N) throw std::runtime_error("set_random_levels: length differs from the number of data rows");
+    host.max_m = opt.max_m;
+    host.max_m0 = opt.max_m0;
+    host.M = opt.max_m;
+    host.ef_construction = opt.ef_construction;
+    host.mult = opt.level_mult;
+    host.set_levels(levels, n);
+    host.layout_links();
+    host.labelled = false;
+    host.labels.clear();
+    have_levels = true;
+    have_graph = false;
+    if (has_device) upload_structure();
+  }
+
+  // ---- slots -----------------------------------------------------------------------------
+  void ensure_pool(int slots, int cand_glob_cap) {
+    const int words = (host.N + 31) / 32;
+    const int undo_cap = std::min(32768, std::max(host.N, 64));
+    if (slots <= pool_slots && words == pool.bitmap_words && cand_glob_cap <= pool.cand_glob_cap && undo_cap == pool.undo_cap)
+      return;
+    slots = std::max(slots, pool_slots);
+    cand_glob_cap = std::max(cand_glob_cap, pool.cand_glob_cap);
+    d_bitmaps.release();
+    d_bitmaps.reserve((size_t)slots * words);
+    HIP_CHECK(hipMemsetAsync(d_bitmaps.p, 0, (size_t)slots * words * 4, stream));
+    d_undo.reserve((size_t)slots * undo_cap);
+    d_cand_glob.reserve((size_t)slots * cand_glob_cap);
+    pool.bitmaps = d_bitmaps.p;
+    pool.bitmap_words = words;
+    pool.undo = d_undo.p;
+    pool.undo_cap = undo_cap;
+    pool.cand_glob = d_cand_glob.p;
+    pool.cand_glob_cap = cand_glob_cap;
+    pool_slots = slots;
+  }
+  // a failed kernel may leave bits set: start over with clean bitmaps
+  void scrub_pool() {
+    HIP_CHECK(hipMemsetAsync(d_bitmaps.p, 0, (size_t)pool_slots * pool.bitmap_words * 4, stream));
+  }
+
+  int auto_cand_lds(int ef, int floor_entries, size_t fixed_bytes) const {
+    if (cand_lds_override > 0) return std::max(cand_lds_override, floor_entries);
+    const size_t budget = 10240;  // ~16 resident wavefronts per CU out of 160 KB LDS
+    size_t used = fixed_bytes + (size_t)(ef + 1) * 8;
+    int c = used < budget ? (int)((budget - used) / 8) : 0;
+    return std::max(c, std::max(floor_entries, 128));
+  }
+
+  template <typename K>
+  int resident_slots(K kernel, size_t lds) const {
+    int per_cu = 0;
+    HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 64, lds));
+    per_cu = std::max(1, std::min(per_cu, 32));
+    return per_cu * num_cus;
+  }
+
+  // ---- search ------------------------------------------------------------------------------
+  template <int DT, int QR>
+  void launch_search(const DevIndex& ix, SearchArgs& a, int max_slots_override, float* ms) {
+    const LdsPlan lp = plan_lds(QR, ix.Dp, a.ef, a.cand_lds, a.lcap, 0, 0);
+    auto kernel = search_kernel<DT, QR>;
+    int slots = resident_slots(kernel, lp.total);
+    if (max_slots_override > 0) slots = max_slots_override;
+    slots = std::max(1, std::min(slots, a.nq));
+    int glob_cap = std::max(4096, 8 * a.ef);
+    for (int attempt = 0; attempt < 6; ++attempt) {
+      ensure_pool(slots, glob_cap);
+      a.pool = pool;
+      a.counter = d_ctl.p;
+      a.status = d_ctl.p + 1;
+      HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 4 * sizeof(int), stream));
+      HIP_CHECK(hipEventRecord(ev0, stream));
+      hipLaunchKernelGGL(kernel, dim3(slots), dim3(64), lp.total, stream, ix, a);
+      HIP_CHECK(hipGetLastError());
+      HIP_CHECK(hipEventRecord(ev1, stream));
+      int ctl[2];
+      HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+      if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
+      if (ctl[1] == 0) return;
+      scrub_pool();
+      glob_cap *= 4;  // a candidate queue overflowed its global area: retry with more room
+    }
+    throw std::runtime_error("search: candidate queue overflow");
+  }
+
+  void search_device(const float* d_qdata, int nq, int k, int ef, int* d_nns_out, float* d_dist_out, int* d_found_out,
+                     int* d_stats, float* ms) {
+    need_device();
+    if (!have_graph) throw std::runtime_error("search_knn: no index (call build_graph or load_index first)");
+    if (nq <= 0) return;
+    if (k <= 0) throw std::runtime_error("search_knn: topk must be positive");
+    ef = std::max(ef, k);
+    DevIndex ix = dev_index();
+    SearchArgs a{};
+    a.q = d_qdata; a.nq = nq; a.k = k; a.ef = ef;
+    a.nns = d_nns_out; a.dists = d_dist_out; a.found = d_found_out; a.stats = d_stats;
+    a.hnswlib_dist = hnswlib_dist;
+    a.lcap = (std::max(std::max(host.S0, host.SU), std::max(k, 64)) + 63) / 64 * 64;
+    const int q = qr();
+    size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
+    a.cand_lds = auto_cand_lds(ef, std::max(k, 64), fixed);
+#define CUHNSW_DISPATCH_SEARCH(DT)                                             \
+  switch (q) {                                                                 \
+    case 1: launch_search<DT, 1>(ix, a, search_slots, ms); break;              \
+    case 2: launch_search<DT, 2>(ix, a, search_slots, ms); break;              \
+    case 4: launch_search<DT, 4>(ix, a, search_slots, ms); break;              \
+    default: launch_search<DT, 0>(ix, a, search_slots, ms); break;             \
+  }
+    if (dist_type == DIST_DOT) { CUHNSW_DISPATCH_SEARCH(DIST_DOT) } else { CUHNSW_DISPATCH_SEARCH(DIST_L2) }
+#undef CUHNSW_DISPATCH_SEARCH
+  }
+
+  void search_host(const float* q, int nq, int k, int ef, int* nns, float* dists, int* found) {
+    need_device();
+    if (nq <= 0) return;
+    if (!q || !nns || !dists || !found) throw std::runtime_error("search_knn: null argument");
+    if (k <= 0) throw std::runtime_error("search_knn: topk must be positive");
+    d_q.reserve((size_t)nq * host.D);
+    d_nns.reserve((size_t)nq * k);
+    d_dist.reserve((size_t)nq * k);
+    d_found.reserve((size_t)nq);
+    HIP_CHECK(hipMemcpyAsync(d_q.p, q, (size_t)nq * host.D * 4, hipMemcpyHostToDevice, stream));
+    search_device(d_q.p, nq, k, ef, d_nns.p, d_dist.p, d_found.p, nullptr, nullptr);
+    HIP_CHECK(hipMemcpyAsync(nns, d_nns.p, (size_t)nq * k * 4, hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipMemcpyAsync(dists, d_dist.p, (size_t)nq * k * 4, hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipMemcpyAsync(found, d_found.p, (size_t)nq * 4, hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+  }
+
+  // ---- build ---------------------------------------------------------------------------------
+  template <int DT, int QR>
+  void build_levels() {
+    const int N = host.N;
+    const int cap_in = 32;
+    const int bmax = std::max(1, build_batch);
+    DevBuf<float> d_dists0, d_distsU, d_sel_keys;
+    DevBuf<uint32_t> d_sel_ids, d_dirty;
+    DevBuf<int> d_sel_cnt, d_inbox_cnt, d_level_nodes;
+    DevBuf<HeapEnt> d_inbox;
+    const int m_cap_max = std::max(host.max_m, host.max_m0);
+    d_dists0.reserve((size_t)N * host.S0);
+    d_distsU.reserve(std::max<size_t>((size_t)host.upper_rows * host.SU, 1));
+    d_sel_ids.reserve((size_t)bmax * m_cap_max);
+    d_sel_keys.reserve((size_t)bmax * m_cap_max);
+    d_sel_cnt.reserve((size_t)bmax);
+    d_dirty.reserve((size_t)bmax * m_cap_max);
+    d_inbox.reserve((size_t)N * cap_in);
+    d_inbox_cnt.reserve((size_t)N);
+    HIP_CHECK(hipMemsetAsync(d_inbox_cnt.p, 0, (size_t)N * 4, stream));
+    HIP_CHECK(hipMemsetAsync(d_links0.p, 0xFF, (size_t)N * host.S0 * 4, stream));
+    if (host.upper_rows > 0) HIP_CHECK(hipMemsetAsync(d_linksU.p, 0xFF, (size_t)host.upper_rows * host.SU * 4, stream));
+
+    // ascending node lists of the upper levels, concatenated
+    std::vector<std::vector<int>> lists(host.maxlevel + 1);
+    for (int i = 0; i < N; ++i)
+      for (int l = 1; l <= host.levels[i]; ++l) lists[l].push_back(i);
+    std::vector<size_t> list_off(host.maxlevel + 2, 0);
+    std::vector<int> flat;
+    for (int l = 1; l <= host.maxlevel; ++l) {
+      list_off[l] = flat.size();
+      flat.insert(flat.end(), lists[l].begin(), lists[l].end());
+    }
+    d_level_nodes.reserve(std::max<size_t>(flat.size(), 1));
+    if (!flat.empty()) HIP_CHECK(hipMemcpyAsync(d_level_nodes.p, flat.data(), flat.size() * 4, hipMemcpyHostToDevice, stream));
+
+    DevIndex ix = dev_index(d_dists0.p, d_distsU.p);
+    auto k_search = build_search_kernel<DT, QR>;
+    auto k_reverse = reverse_kernel<DT, QR>;
+    const int efc = opt.ef_construction;
+    const int glob_cap = std::max(4096, 8 * efc);
+
+    for (int lv = host.maxlevel; lv >= 0; --lv) {
+      const int n_lv = lv == 0 ? N : (int)lists[lv].size();
+      const int* nodes = lv == 0 ? nullptr : d_level_nodes.p + list_off[lv];
+      const int S = lv == 0 ? host.S0 : host.SU;
+      const int m_cap = lv == 0 ? host.max_m0 : host.max_m;
+      int n_skel = 0;
+      if (lv < host.maxlevel) {
+        n_skel = (int)lists[lv + 1].size();
+        long long work = (long long)n_skel * S;
+        hipLaunchKernelGGL(inherit_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, ix, lv,
+                           d_level_nodes.p + list_off[lv + 1], n_skel);
+        HIP_CHECK(hipGetLastError());
+      }
+      BuildArgs a{};
+      a.level = lv;
+      a.level_nodes = nodes;
+      a.efc = efc;
+      a.m_cap = m_cap;
+      a.nn_num = (int)(m_cap * opt.heuristic_coef);
+      a.save_remains = opt.save_remains ? 1 : 0;
+      a.sel_ids = d_sel_ids.p; a.sel_keys = d_sel_keys.p; a.sel_cnt = d_sel_cnt.p;
+      a.counter = d_ctl.p; a.status = d_ctl.p + 1;
+      a.inbox = d_inbox.p; a.inbox_cnt = d_inbox_cnt.p; a.cap_in = cap_in;
+      a.dirty = d_dirty.p; a.dirty_cnt = d_ctl.p + 2;
+      a.lcap = (std::max(S, 64) + 63) / 64 * 64;
+      const int q = QR;
+      size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_cap * 8 + 64 +
+                     (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
+      a.cand_lds = auto_cand_lds(efc, 64, fixed);
+      const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_cap);
+      const LdsPlan lp3 = plan_lds(QR, Dp, S + cap_in, 0, a.lcap, S + cap_in, m_cap);
+      const int slots1 = resident_slots(k_search, lp1.total);
+      const int slots3 = resident_slots(k_reverse, lp3.total);
+      ensure_pool(slots1, glob_cap);
+      a.pool = pool;
+
+      int pos = 0;
+      while (pos < n_lv) {
+        int b = std::max(1, std::min(bmax, (n_skel + pos) / 4));
+        b = std::min(b, n_lv - pos);
+        a.begin = pos;
+        a.count = b;
+        // counter and dirty count back to zero; the status word is sticky
+        HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, sizeof(int), stream));
+        HIP_CHECK(hipMemsetAsync(d_ctl.p + 2, 0, sizeof(int), stream));
+        hipLaunchKernelGGL(k_search, dim3(std::min(b, slots1)), dim3(64), lp1.total, stream, ix, a);
+        HIP_CHECK(hipGetLastError());
+        long long work = (long long)b * m_cap;
+        hipLaunchKernelGGL(apply_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, ix, a);
+        HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(k_reverse, dim3((unsigned)std::min<long long>(work, slots3)), dim3(64), lp3.total, stream, ix, a);
+        HIP_CHECK(hipGetLastError());
+        pos += b;
+      }
+    }
+    int ctl[4];
+    HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+    if (ctl[1] != 0) {
+      scrub_pool();
+      throw std::runtime_error("build_graph: candidate queue overflow");
+    }
+  }
+
+  void build_graph() {
+    need_device();
+    if (!have_data || !have_levels) throw std::runtime_error("build_graph: call set_data and set_random_levels first");
+    HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 4 * sizeof(int), stream));
+    HIP_CHECK(hipStreamSynchronize(stream));
+    auto t0 = std::chrono::steady_clock::now();
+    const int q = qr();
+#define CUHNSW_DISPATCH_BUILD(DT)               \
+  switch (q) {                                  \
+    case 1: build_levels<DT, 1>(); break;       \
+    case 2: build_levels<DT, 2>(); break;       \
+    case 4: build_levels<DT, 4>(); break;       \
+    default: build_levels<DT, 0>(); break;      \
+  }
+    if (dist_type == DIST_DOT) { CUHNSW_DISPATCH_BUILD(DIST_DOT) } else { CUHNSW_DISPATCH_BUILD(DIST_L2) }
+#undef CUHNSW_DISPATCH_BUILD
+    last_build_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    have_graph = true;
+    host_links_stale = true;
+  }
+
+  // ---- index file --------------------------------------------------------------------------------
+  void save_index(const char* path) {
+    if (!have_graph) throw std::runtime_error("save_index: no index to save");
+    if (host_links_stale) download_links();
+    write_index_file(host, path);
+  }
+  void load_index(const char* path) {
+    HostIndex fresh;
+    read_index_file(fresh, path);
+    if (fresh.N <= 0) throw std::runtime_error("load_index: empty index");
+    host = std::move(fresh);
+    have_data = have_levels = have_graph = true;
+    host_links_stale = false;
+    if (has_device) {
+      upload_vectors();
+      upload_structure();
+      upload_links();
+      d_labels.reserve((size_t)host.N);
+      HIP_CHECK(hipMemcpyAsync(d_labels.p, host.labels.data(), (size_t)host.N * 8, hipMemcpyHostToDevice, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+      pool_slots = 0;  // N may have changed: rebuild the slot pool lazily
+      pool = SlotPool{};
+    }
+  }
+};
+
+}  // namespace cuhnsw_amd
+
+// ---------------------------------------------------------------------------------------------- C ABI
+using cuhnsw_amd::Engine;
+
+struct cuhnsw_engine {
+  Engine impl;
+};
+
+namespace {
+thread_local std::string g_create_error;
+
+template <typename F>
+int guarded(cuhnsw_engine* e, F&& f) {
+  if (!e) return -1;
+  try {
+    e->impl.err.clear();
+    f(e->impl);
+    return 0;
+  } catch (const std::exception& ex) {
+    e->impl.err = ex.what();
+    return -1;
+  } catch (...) {
+    e->impl.err = "unknown error";
+    return -1;
+  }
+}
+}  // namespace
+
+extern "C" {
+
+int cuhnsw_create(cuhnsw_engine** out) {
+  if (!out) return -1;
+  try {
+    *out = new cuhnsw_engine();
+    return 0;
+  } catch (const std::exception& ex) {
+    g_create_error = ex.what();
+    *out = nullptr;
+    return -1;
+  }
+}
+void cuhnsw_destroy(cuhnsw_engine* e) { delete e; }
+const char* cuhnsw_last_error(cuhnsw_engine* e) { return e ? e->impl.err.c_str() : g_create_error.c_str(); }
+
+int cuhnsw_init(cuhnsw_engine* e, const char* opt_path) {
+  if (!e) return -1;
+  int rc = e->impl.init(opt_path);
+  if (rc == 1) e->impl.err = std::string("cannot read or parse option file: ") + (opt_path ? opt_path : "(null)");
+  if (rc == 2) e->impl.err = "invalid dist type " + e->impl.opt.dist_type;
+  return rc;
+}
+int cuhnsw_set_data(cuhnsw_engine* e, const float* data, int num_data, int num_dims) {
+  return guarded(e, [&](Engine& g) { g.set_data(data, num_data, num_dims); });
+}
+int cuhnsw_set_random_levels(cuhnsw_engine* e, const int* levels, int num_levels) {
+  return guarded(e, [&](Engine& g) {
+    if (!levels) throw std::runtime_error("set_random_levels: null levels");
+    g.set_random_levels(levels, num_levels);
+  });
+}
+int cuhnsw_build_graph(cuhnsw_engine* e) { return guarded(e, [&](Engine& g) { g.build_graph(); }); }
+int cuhnsw_save_index(cuhnsw_engine* e, const char* fpath) {
+  return guarded(e, [&](Engine& g) { g.save_index(fpath ? fpath : ""); });
+}
+int cuhnsw_load_index(cuhnsw_engine* e, const char* fpath) {
+  return guarded(e, [&](Engine& g) { g.load_index(fpath ? fpath : ""); });
+}
+int cuhnsw_search_knn(cuhnsw_engine* e, const float* qdata, int num_queries, int topk, int ef_search, int* nns,
+                      float* distances, int* found_cnt) {
+  return guarded(e, [&](Engine& g) { g.search_host(qdata, num_queries, topk, ef_search, nns, distances, found_cnt); });
+}
+int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search, int* d_nns,
+                             float* d_distances, int* d_found_cnt, int* d_stats, float* kernel_ms) {
+  return guarded(e, [&](Engine& g) {
+    g.search_device(d_qdata, num_queries, topk, ef_search, d_nns, d_distances, d_found_cnt, d_stats, kernel_ms);
+  });
+}
+int cuhnsw_num_data(cuhnsw_engine* e) { return e ? e->impl.host.N : 0; }
+int cuhnsw_num_dims(cuhnsw_engine* e) { return e ? e->impl.host.D : 0; }
+int cuhnsw_max_level(cuhnsw_engine* e) { return e ? e->impl.host.maxlevel : 0; }
+int cuhnsw_enter_point(cuhnsw_engine* e) { return e ? (int)e->impl.host.enterpoint : 0; }
+int cuhnsw_has_device(void) { return cuhnsw_amd::device_present() ? 1 : 0; }
+double cuhnsw_last_build_seconds(cuhnsw_engine* e) { return e ? e->impl.last_build_seconds : 0.0; }
+int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
+  if (!e || !name) return -1;
+  std::string n(name);
+  if (n == "build_batch") e->impl.build_batch = (int)value;
+  else if (n == "search_slots") e->impl.search_slots = (int)value;
+  else if (n == "cand_lds") e->impl.cand_lds_override = (int)value;
+  else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
+  else return -1;
+  return 0;
+}
+
+}  // extern "C"

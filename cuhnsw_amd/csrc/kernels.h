@@ -1,0 +1,438 @@
+// The launched kernels: batch search, and the three phases of a build batch.
+//
+// search_kernel        replaces GetEntryPointsKernel + SearchGraphKernel
+//                      (cpp/include/cuda_search_kernels.cuh:11-165 in the reference):
+//                      one launch does the descent through every upper level and the
+//                      level-0 ef-search for a whole query batch.
+// build_search_kernel, apply_kernel, reverse_kernel
+//                      replace BuildLevelGraphKernel + SearchHeuristic
+//                      (cpp/include/cuda_build_kernels.cuh:68-338).  The reference
+//                      inserts all nodes of a level concurrently under per-node spin
+//                      locks; here a level is inserted in batches of three lock-free
+//                      phases separated by kernel boundaries:
+//                        1. every node of the batch searches the frozen graph and
+//                           selects its neighbours (read-only on the graph),
+//                        2. the selections are written and each chosen neighbour y
+//                           receives the newcomer in y's inbox,
+//                        3. one wavefront per touched y merges inbox and row (append
+//                           while there is room, else the selection heuristic).
+//                      The result is deterministic for a given batch schedule.
+#pragma once
+#include "device_core.h"
+
+namespace cuhnsw_amd {
+
+struct SlotPool {
+  uint32_t* bitmaps;
+  int bitmap_words;
+  uint32_t* undo;
+  int undo_cap;
+  HeapEnt* cand_glob;
+  int cand_glob_cap;
+};
+
+struct SearchArgs {
+  const float* q;  // nq x D
+  int nq, k, ef;
+  int* nns;
+  float* dists;
+  int* found;
+  int* stats;    // nq x 4 or null
+  int* counter;  // work queue head
+  int* status;   // set to 1 when a candidate queue ran out of room
+  SlotPool pool;
+  int cand_lds, lcap, hnswlib_dist;
+};
+
+struct BuildArgs {
+  int level;
+  const int* level_nodes;  // ascending ids of the nodes of this level, null = identity
+  int begin, count;        // batch = level_nodes[begin .. begin+count)
+  int efc, m_cap, nn_num, save_remains;
+  uint32_t* sel_ids;  // count x m_cap
+  float* sel_keys;
+  int* sel_cnt;
+  int* counter;
+  int* status;
+  SlotPool pool;
+  int cand_lds, lcap;
+  HeapEnt* inbox;  // N x cap_in
+  int* inbox_cnt;  // N
+  int cap_in;
+  uint32_t* dirty;
+  int* dirty_cnt;
+};
+
+__host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
+
+// LDS layout of one wavefront (shared by host sizing and device carving)
+struct LdsPlan {
+  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, total;
+};
+__host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds, int lcap, int n_sorted, int n_out) {
+  LdsPlan p;
+  size_t o = 0;
+  p.qlds = o;
+  if (qr == 0) o += (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16;
+  p.top = o; o = align16(o + (size_t)(ef + 1) * 8);
+  p.cand = o; o = align16(o + (size_t)cand_lds * 8);
+  p.sorted_id = o; o = align16(o + (size_t)n_sorted * 4);
+  p.sorted_key = o; o = align16(o + (size_t)n_sorted * 4);
+  p.out_id = o; o = align16(o + (size_t)n_out * 4);
+  p.out_key = o; o = align16(o + (size_t)n_out * 4);
+  p.nbuf = o; o = align16(o + (size_t)lcap * 4);
+  p.dbuf = o; o = align16(o + (size_t)lcap * 4);
+  p.total = o;
+  return p;
+}
+
+__device__ __forceinline__ void bind_slot(Scratch& s, const SlotPool& pool, int slot) {
+  s.bitmap = pool.bitmaps + (size_t)slot * pool.bitmap_words;
+  s.bitmap_words = pool.bitmap_words;
+  s.undo = pool.undo + (size_t)slot * pool.undo_cap;
+  s.undo_cap = pool.undo_cap;
+  s.cand_glob = pool.cand_glob + (size_t)slot * pool.cand_glob_cap;
+  s.cand_glob_cap = pool.cand_glob_cap;
+}
+
+template <int DT, int QR>
+__global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x;
+  const LdsPlan lp = plan_lds(QR, ix.Dp, a.ef, a.cand_lds, a.lcap, 0, 0);
+  Scratch s;
+  s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
+  s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
+  s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
+  s.cand_lds = a.cand_lds;
+  s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
+  s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
+  bind_slot(s, a.pool, blockIdx.x);
+
+  for (;;) {
+    int qi = 0;
+    if (lane == 0) qi = atomicAdd(a.counter, 1);
+    qi = __builtin_amdgcn_readfirstlane(qi);
+    if (qi >= a.nq) break;
+    QVec<QR> qv;
+    load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
+    SearchState st;
+    st.top_size = 0; st.cand_size = 0; st.lower = 0.f; st.undo_cnt = 0;
+    st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
+
+    uint32_t cur = ix.enterpoint;
+    float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
+    descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
+
+    visit_single(s, st, cur, lane);
+    if (lane == 0) s.nbuf[0] = cur;
+    __syncthreads();
+    search_level<DT, QR, false>(ix, qv, 0, a.ef, s, st, 1, lane);
+
+    // keep the k best (literal pops), then order them by (key, label) ascending as
+    // hnswlib's result queue does
+    if (lane == 0) {
+      LdsHeap top{s.top};
+      while (st.top_size > a.k) heap_pop<false>(top, st.top_size);
+    }
+    const int T = __builtin_amdgcn_readfirstlane(st.top_size);
+    __syncthreads();
+    uint64_t* tie = nullptr;
+    if (ix.labels) {
+      tie = reinterpret_cast<uint64_t*>(s.cand);
+      for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
+      __syncthreads();
+    }
+    rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
+    __syncthreads();
+    if (!a.hnswlib_dist && T > 0) {
+      dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
+      __syncthreads();
+    }
+    for (int r = lane; r < a.k; r += 64) {
+      int out_id = -1;
+      float out_d = INFINITY;
+      if (r < T) {
+        uint32_t id = s.nbuf[r];
+        out_id = ix.labels ? (int)ix.labels[id] : (int)id;
+        out_d = s.dbuf[r];
+      }
+      a.nns[(size_t)qi * a.k + r] = out_id;
+      a.dists[(size_t)qi * a.k + r] = out_d;
+    }
+    if (lane == 0) {
+      a.found[qi] = st.fail ? -1 : T;
+      if (st.fail) *a.status = 1;
+      if (a.stats) {
+        a.stats[(size_t)qi * 4 + 0] = st.n_dist;
+        a.stats[(size_t)qi * 4 + 1] = st.n_hops;
+        a.stats[(size_t)qi * 4 + 2] = st.n_dist_upper;
+        a.stats[(size_t)qi * 4 + 3] = st.n_sweeps;
+      }
+    }
+    undo_visited(s, st, lane);
+    __syncthreads();
+  }
+}
+
+// loads the (zero padded, 128-byte aligned) vector of a stored node as the "query"
+template <int QR>
+__device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, const DevIndex& ix, uint32_t node, int lane) {
+  const int rowlen = ix.Dp >> 2;
+  const float4* p = reinterpret_cast<const float4*>(ix.vectors) + (size_t)node * rowlen;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (QR > 0) {
+    const int sub = lane & 15;
+#pragma unroll
+    for (int k = 0; k < (QR > 0 ? QR : 1); ++k) qv.q[k] = (sub + 16 * k < rowlen) ? p[sub + 16 * k] : zero;
+  } else {
+    const int chunks = (rowlen + 15) / 16 * 16;
+    __syncthreads();
+    for (int c = lane; c < chunks; c += 64) qlds[c] = c < rowlen ? p[c] : zero;
+    __syncthreads();
+  }
+}
+
+// Neighbour selection (HNSW Alg. 4 / hnswlib getNeighborsByHeuristic2) with the two
+// extras of the reference's SearchHeuristic (cpp/include/cuda_build_kernels.cuh:68-162):
+// the first nn_num candidates pass unconditionally, and with save_remains pruned
+// candidates fill the row from the tail.  Candidates sid/skey[0..T) are ascending.
+// Returns the degree; oid/okey[0..degree) is the new row.
+template <int DT, int QR>
+__device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32_t* sid, const float* skey, int T, int m,
+                                                int nn_num, int save_remains, uint32_t* oid, float* okey, Scratch& s,
+                                                int lane) {
+  int head = 0;
+  int tail = (m < T ? m : T) - 1;
+  const int max_head = tail + 1;
+  for (int j = 0; j < T; ++j) {
+    if (head >= m) break;
+    const uint32_t c = sid[j];
+    const float dq = skey[j];
+    bool skip = false;
+    if (head >= nn_num && head > 0) {
+      QVec<QR> cv;
+      load_node_query<QR>(cv, s.qlds, ix, c, lane);
+      dist_list<DT, QR, false>(ix, cv, s.qlds, oid, head, s.dbuf, lane);
+      __syncthreads();
+      bool mine = false;
+      for (int t = lane; t < head; t += 64) mine = mine || (dq > s.dbuf[t]);
+      skip = __ballot(mine) != 0ull;
+      __syncthreads();
+    }
+    if (!skip) {
+      if (lane == 0) { oid[head] = c; okey[head] = dq; }
+      head++;
+    } else if (tail >= head) {
+      if (lane == 0) { oid[tail] = c; okey[tail] = dq; }
+      tail--;
+    }
+    __syncthreads();
+  }
+  return save_remains ? max_head : head;
+}
+
+// Phase 1 of a build batch: search + select, read-only on the graph.
+template <int DT, int QR>
+__global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x;
+  const LdsPlan lp = plan_lds(QR, ix.Dp, a.efc, a.cand_lds, a.lcap, a.efc, a.m_cap);
+  Scratch s;
+  s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
+  s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
+  s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
+  s.cand_lds = a.cand_lds;
+  s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
+  s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
+  uint32_t* sid = reinterpret_cast<uint32_t*>(smem + lp.sorted_id);
+  float* skey = reinterpret_cast<float*>(smem + lp.sorted_key);
+  uint32_t* oid = reinterpret_cast<uint32_t*>(smem + lp.out_id);
+  float* okey = reinterpret_cast<float*>(smem + lp.out_key);
+  bind_slot(s, a.pool, blockIdx.x);
+
+  for (;;) {
+    int b = 0;
+    if (lane == 0) b = atomicAdd(a.counter, 1);
+    b = __builtin_amdgcn_readfirstlane(b);
+    if (b >= a.count) break;
+    const uint32_t x = a.level_nodes ? (uint32_t)a.level_nodes[a.begin + b] : (uint32_t)(a.begin + b);
+    QVec<QR> qv;
+    load_node_query<QR>(qv, s.qlds, ix, x, lane);
+    SearchState st;
+    st.top_size = 0; st.cand_size = 0; st.lower = 0.f; st.undo_cnt = 0;
+    st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
+    visit_single(s, st, x, lane);  // a node never links to itself
+
+    int n_seed = 0;
+    if (ix.levels[x] == a.level) {
+      // first appearance of x: enter through the finished upper levels
+      if (a.level == ix.maxlevel) {
+        if (x != ix.enterpoint) {
+          visit_single(s, st, ix.enterpoint, lane);
+          if (lane == 0) s.nbuf[0] = ix.enterpoint;
+          n_seed = 1;
+        }
+      } else {
+        uint32_t cur = ix.enterpoint;
+        float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
+        descend<DT, QR>(ix, qv, ix.maxlevel, a.level, cur, dcur, s, st, lane);
+        visit_single(s, st, cur, lane);
+        if (lane == 0) s.nbuf[0] = cur;
+        n_seed = 1;
+      }
+    } else {
+      // x also lives above: start from the links it inherited at this level
+      n_seed = visit_row(link_row(ix, x, a.level), row_stride(ix, a.level), s, st, lane);
+    }
+    __syncthreads();
+    search_level<DT, QR, true>(ix, qv, a.level, a.efc, s, st, n_seed, lane);
+
+    const int T = st.top_size;
+    rank_sort(s.top, nullptr, T, sid, skey, lane);
+    __syncthreads();
+    const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);
+    for (int j = lane; j < a.m_cap; j += 64) {
+      a.sel_ids[(size_t)b * a.m_cap + j] = j < deg ? oid[j] : kEmpty;
+      a.sel_keys[(size_t)b * a.m_cap + j] = j < deg ? okey[j] : 0.f;
+    }
+    if (lane == 0) {
+      a.sel_cnt[b] = deg;
+      if (st.fail) *a.status = 1;
+    }
+    undo_visited(s, st, lane);
+    __syncthreads();
+  }
+}
+
+__device__ __forceinline__ uint32_t* link_row_mut(const DevIndex& ix, uint32_t node, int level) {
+  return level == 0 ? ix.links0 + (size_t)node * ix.S0 : ix.linksU + (size_t)(ix.upper_off[node] + level - 1) * ix.SU;
+}
+__device__ __forceinline__ float* dist_row_mut(const DevIndex& ix, uint32_t node, int level) {
+  return level == 0 ? ix.dists0 + (size_t)node * ix.S0 : ix.distsU + (size_t)(ix.upper_off[node] + level - 1) * ix.SU;
+}
+
+// Phase 2: write the selected rows and post the reverse links.
+__global__ void __launch_bounds__(256) apply_kernel(DevIndex ix, BuildArgs a) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long long)a.count * a.m_cap) return;
+  const int b = (int)(i / a.m_cap), j = (int)(i % a.m_cap);
+  const uint32_t x = a.level_nodes ? (uint32_t)a.level_nodes[a.begin + b] : (uint32_t)(a.begin + b);
+  const int deg = a.sel_cnt[b];
+  const uint32_t y = j < deg ? a.sel_ids[i] : kEmpty;
+  const float key = a.sel_keys[i];
+  link_row_mut(ix, x, a.level)[j] = y;
+  dist_row_mut(ix, x, a.level)[j] = key;
+  if (j < deg) {
+    int slot = atomicAdd(&a.inbox_cnt[y], 1);
+    if (slot < a.cap_in) {
+      HeapEnt e;
+      e.key = key;
+      e.id = x;
+      a.inbox[(size_t)y * a.cap_in + slot] = e;
+    }
+    if (slot == 0) a.dirty[atomicAdd(a.dirty_cnt, 1)] = y;
+  }
+}
+
+// Phase 3: one wavefront per node that received reverse links.
+template <int DT, int QR>
+__global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x;
+  const int S = row_stride(ix, a.level);
+  const int ncand = S + a.cap_in;
+  // plan: "top" region holds the merged candidates, sorted_* their ranking
+  const LdsPlan lp = plan_lds(QR, ix.Dp, ncand, 0, a.lcap, ncand, a.m_cap);
+  Scratch s;
+  s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
+  HeapEnt* cbuf = reinterpret_cast<HeapEnt*>(smem + lp.top);
+  s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
+  s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
+  uint32_t* sid = reinterpret_cast<uint32_t*>(smem + lp.sorted_id);
+  float* skey = reinterpret_cast<float*>(smem + lp.sorted_key);
+  uint32_t* oid = reinterpret_cast<uint32_t*>(smem + lp.out_id);
+  float* okey = reinterpret_cast<float*>(smem + lp.out_key);
+  const int n_dirty = *a.dirty_cnt;
+
+  for (int di = blockIdx.x; di < n_dirty; di += gridDim.x) {
+    const uint32_t y = a.dirty[di];
+    int nin = a.inbox_cnt[y];
+    nin = nin < a.cap_in ? nin : a.cap_in;
+    uint32_t* row = link_row_mut(ix, y, a.level);
+    float* drow = dist_row_mut(ix, y, a.level);
+    // existing links
+    int n0 = 0;
+    for (int base = 0; base < S; base += 64) {
+      uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
+      float key = (base + lane < S) ? drow[base + lane] : 0.f;
+      bool valid = id != kEmpty;
+      unsigned long long mask = __ballot(valid);
+      int pos = n0 + __popcll(mask & ((1ull << lane) - 1ull));
+      if (valid) { cbuf[pos].key = key; cbuf[pos].id = id; }
+      n0 += __popcll(mask);
+    }
+    __syncthreads();
+    // newcomers that are not linked yet
+    int T = n0;
+    for (int base = 0; base < nin; base += 64) {
+      HeapEnt e;
+      e.key = 0.f; e.id = kEmpty;
+      bool keep = false;
+      if (base + lane < nin) {
+        e = a.inbox[(size_t)y * a.cap_in + base + lane];
+        keep = true;
+        for (int t = 0; t < n0; ++t) keep = keep && (cbuf[t].id != e.id);
+      }
+      unsigned long long mask = __ballot(keep);
+      int pos = T + __popcll(mask & ((1ull << lane) - 1ull));
+      if (keep) cbuf[pos] = e;
+      T += __popcll(mask);
+    }
+    __syncthreads();
+    const int n_new = T - n0;
+    if (n_new > 0) {
+      if (T <= a.m_cap) {
+        // room for all: append the newcomers, ordered by (key, id)
+        rank_sort(cbuf + n0, nullptr, n_new, sid, skey, lane);
+        __syncthreads();
+        for (int t = lane; t < n_new; t += 64) {
+          row[n0 + t] = sid[t];
+          drow[n0 + t] = skey[t];
+        }
+      } else {
+        rank_sort(cbuf, nullptr, T, sid, skey, lane);
+        __syncthreads();
+        const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);
+        for (int j = lane; j < a.m_cap; j += 64) {
+          row[j] = j < deg ? oid[j] : kEmpty;
+          drow[j] = j < deg ? okey[j] : 0.f;
+        }
+      }
+    }
+    if (lane == 0) a.inbox_cnt[y] = 0;
+    __syncthreads();
+  }
+}
+
+// Start of a level: every node that also lives on level+1 inherits its links from there
+// (the reference does the same on the host, cpp/src/cuhnsw_build.cu:113-125; here the
+// link keys travel with the ids).
+__global__ void __launch_bounds__(256) inherit_kernel(DevIndex ix, int level, const int* upper_nodes, int count) {
+  const int S = level == 0 ? ix.S0 : ix.SU;
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long long)count * S) return;
+  const uint32_t x = (uint32_t)upper_nodes[i / S];
+  const int j = (int)(i % S);
+  const size_t src = (size_t)(ix.upper_off[x] + level) * ix.SU;  // row of level + 1
+  uint32_t id = kEmpty;
+  float key = 0.f;
+  if (j < ix.SU) {
+    id = ix.linksU[src + j];
+    key = ix.distsU[src + j];
+  }
+  link_row_mut(ix, x, level)[j] = id;
+  dist_row_mut(ix, x, level)[j] = key;
+}
+
+}  // namespace cuhnsw_amd

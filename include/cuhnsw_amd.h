@@ -1,0 +1,109 @@
+/* C ABI of the MI355X-native HNSW engine (libcuhnsw_amd.so).
+ *
+ * Every entry point is what a foreign-function binding of the reference's hot
+ * path would bind: one call per method of the reference's host class
+ * cuhnsw::CuHNSW (cpp/include/cuhnsw.hpp:61-71 in js1010/cuhnsw), which the
+ * reference exposes to Python through CuHNSWBind (cuhnsw/bindings.cc:18-72).
+ * Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - functions returning int: 0 = success, non-zero = failure; the message is
+ *     available from cuhnsw_last_error(engine) (the reference throws
+ *     std::runtime_error instead, cpp/include/cuda_base_kernels.cuh:30-37).
+ *   - an engine is not thread-safe; calls are synchronous.
+ *   - distances: dist_type "dot" -> -<q,x>, "l2" -> squared L2
+ *     (cpp/include/cuda_dist_kernels.cuh:112-124).  Candidates are *ordered* by
+ *     hnswlib's key (1 - <q,x> for "dot") so that ids equal hnswlib's.
+ */
+#ifndef CUHNSW_AMD_H_
+#define CUHNSW_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cuhnsw_engine cuhnsw_engine;
+
+/* cuhnsw::CuHNSW::CuHNSW() (cpp/src/cuhnsw_base.cu:13-16).  Works without a GPU
+ * (host-side calls: init, load_index, save_index, set_random_levels); every call
+ * that needs the device fails with a clear message when none is present. */
+int cuhnsw_create(cuhnsw_engine** out);
+/* cuhnsw::CuHNSW::~CuHNSW() (cpp/src/cuhnsw_base.cu:64) */
+void cuhnsw_destroy(cuhnsw_engine* e);
+/* message of the last failed call on this engine ("" if none) */
+const char* cuhnsw_last_error(cuhnsw_engine* e);
+
+/* bool CuHNSW::Init(std::string opt_path) (cpp/src/cuhnsw_base.cu:67-106):
+ * opt_path names a JSON file holding the option table of
+ * cuhnsw/proto/config.proto:10-26.  Returns 0 on success, 1 if the file cannot be
+ * read or parsed (the reference returns false), 2 on an invalid dist_type (the
+ * reference throws). */
+int cuhnsw_init(cuhnsw_engine* e, const char* opt_path);
+
+/* void CuHNSW::SetData(const float* data, int num_data, int num_dims)
+ * (cpp/src/cuhnsw_base.cu:108-128).  data: row-major float32 [num_data x
+ * num_dims] in host memory.  The engine keeps its own copy (the reference keeps
+ * the caller's raw pointer). */
+int cuhnsw_set_data(cuhnsw_engine* e, const float* data, int num_data, int num_dims);
+
+/* void CuHNSW::SetRandomLevels(const int* levels) (cpp/src/cuhnsw_base.cu:130-156):
+ * levels[i] = number of upper levels of node i; num_levels must equal num_data. */
+int cuhnsw_set_random_levels(cuhnsw_engine* e, const int* levels, int num_levels);
+
+/* void CuHNSW::BuildGraph() (cpp/src/cuhnsw_build.cu:96-102): builds every level
+ * on the GPU; requires set_data + set_random_levels. */
+int cuhnsw_build_graph(cuhnsw_engine* e);
+
+/* void CuHNSW::SaveIndex(std::string fpath) (cpp/src/cuhnsw_base.cu:159-247):
+ * hnswlib index file format. */
+int cuhnsw_save_index(cuhnsw_engine* e, const char* fpath);
+/* void CuHNSW::LoadIndex(std::string fpath) (cpp/src/cuhnsw_base.cu:250-365):
+ * after it, search returns the file's labels instead of internal ids
+ * (cpp/src/cuhnsw_build.cu:284-286). */
+int cuhnsw_load_index(cuhnsw_engine* e, const char* fpath);
+
+/* void CuHNSW::SearchGraph(const float* qdata, int num_queries, int topk,
+ *   int ef_search, int* nns, float* distances, int* found_cnt)
+ * (cpp/src/cuhnsw_build.cu:210-290).  All pointers are host memory, outputs are
+ * caller-allocated: nns int32 [num_queries x topk], distances float32
+ * [num_queries x topk] ascending, found_cnt int32 [num_queries]; only the first
+ * found_cnt[i] entries of a row are defined.  ef_search is raised to topk
+ * (cuhnsw/pyhnsw.py:80 does the same before the call). */
+int cuhnsw_search_knn(cuhnsw_engine* e, const float* qdata, int num_queries, int topk, int ef_search,
+                      int* nns, float* distances, int* found_cnt);
+
+/* Same search with queries and outputs already in device memory (HBM); nothing
+ * is copied.  Counterpart of the kernel launch inside CuHNSW::SearchGraph
+ * (cpp/src/cuhnsw_build.cu:254-275).  d_stats may be null, else int32
+ * [num_queries x 4]: level-0 distance evaluations, level-0 expanded candidates,
+ * upper-level distance evaluations, upper-level sweeps.  The call returns after
+ * the kernel has finished; kernel_ms (may be null) receives the kernel's duration
+ * measured with HIP events on the engine's stream. */
+int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
+                             int* d_nns, float* d_distances, int* d_found_cnt, int* d_stats, float* kernel_ms);
+
+/* Introspection used by bindings, tests and the benchmark (the reference keeps
+ * the same facts in private members num_data_, num_dims_, max_level_,
+ * enter_point_, cpp/include/cuhnsw.hpp:87-108). */
+int cuhnsw_num_data(cuhnsw_engine* e);
+int cuhnsw_num_dims(cuhnsw_engine* e);
+int cuhnsw_max_level(cuhnsw_engine* e);
+int cuhnsw_enter_point(cuhnsw_engine* e);
+/* 1 if a HIP device is usable by this process, else 0 */
+int cuhnsw_has_device(void);
+/* seconds spent inside the last cuhnsw_build_graph (device work, event-timed) */
+double cuhnsw_last_build_seconds(cuhnsw_engine* e);
+/* tuning knobs that are not part of the reference's option table:
+ *   "build_batch"   largest number of nodes inserted per batch (default 16384)
+ *   "search_slots"  resident wavefronts used by search (0 = automatic)
+ *   "cand_lds"      candidate-queue entries kept in LDS (0 = automatic)
+ *   "hnswlib_dist"  1 = return hnswlib distances (1-dot) instead of -dot
+ * returns non-zero for an unknown name */
+int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUHNSW_AMD_H_ */
