@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--no-cpu]
+
+Workload (default C2): the GloVe-50-shaped angular configuration — 1 183 514 x 50
+float32 vectors from the seeded 1000-centre Gaussian mixture, L2-normalised,
+dist_type=dot, max_m=12, max_m0=24, ef_construction=110; 10 000 queries, topk=10,
+ef_search=300.  The index is built on the GPU (build seconds reported); one *step* is
+one search pass of the whole query batch with queries and outputs resident in HBM.
+
+Prints one JSON line: value = search queries/s over the timed steps; `roofline`
+prices the search kernel's algorithmic distance-gather bytes (sum over queries of
+level-0 distance evaluations x 4*D, counted on the device) against the kernel time
+measured with HIP events on the engine's stream; `cpu_baseline` times the CPU oracle
+(hnswlib-semantics search of the same index file, and a bounded CPU build sample) on
+this host's cores.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=20)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--workload", default="C2")
+  ap.add_argument("--n", type=int, default=None, help="shrink the data set (debugging)")
+  ap.add_argument("--nq", type=int, default=None)
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  args = ap.parse_args()
+  if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+    print("bench.py: this build runs on ONE GPU (the index and the query batch live on a single "
+          "device; there is no multi-GPU path) — run with --gpus 1", file=sys.stderr)
+    sys.exit(2)
+
+  import torch  # device buffers only; loaded before the engine so that one HIP runtime is used
+  from cuhnsw_amd import capi, datasets
+  if not torch.cuda.is_available() or not capi.has_device():
+    print("bench.py: no GPU visible", file=sys.stderr)
+    sys.exit(3)
+
+  t0 = time.time()
+  data, queries, spec = datasets.make(args.workload, n=args.n, nq=args.nq)
+  o = dict(spec["opt"])
+  n, d = data.shape
+  nq, k, ef = queries.shape[0], spec["topk"], spec["ef"][-1] if args.workload != "C2" else 300
+  mult = o.get("level_mult") or 1.0 / np.log(o["max_m"])
+  levels = datasets.random_levels(n, mult)
+  gen_s = time.time() - t0
+
+  opt = dict(seed=777, c_log_level=2, py_log_level=2, max_m=o["max_m"], max_m0=o["max_m0"],
+             ef_construction=o["ef_construction"], level_mult=mult, save_remains=False, hyper_threads=10.0,
+             block_dim=32, dist_type=o["dist_type"], visited_table_size=0, visited_list_size=8192, nrz=False,
+             reverse_cand=False, heuristic_coef=0.0)
+  tmpdir = tempfile.mkdtemp(prefix="cuhnsw_bench_")
+  opt_path = os.path.join(tmpdir, "opt.json")
+  with open(opt_path, "w") as f:
+    json.dump(opt, f)
+  eng = capi.Engine()
+  assert eng.init(opt_path) == 0
+  t0 = time.time()
+  eng.set_data(data)
+  upload_s = time.time() - t0
+  eng.set_random_levels(levels)
+  eng.build_graph()                      # warm-up build (first launch pays code loading)
+  eng.set_random_levels(levels)
+  eng.build_graph()
+  build_s = eng.last_build_seconds
+
+  # exact top-k on the GPU (harness only) for recall
+  dd = torch.from_numpy(data).cuda()
+  qq = torch.from_numpy(queries).cuda()
+  gt = []
+  for s in range(0, nq, 500):
+    qs = qq[s:s + 500]
+    if o["dist_type"] == "dot":
+      score = -(qs @ dd.T)
+    else:
+      score = (dd * dd).sum(1)[None, :] - 2.0 * (qs @ dd.T)
+    gt.append(torch.topk(score, k, dim=1, largest=False).indices.cpu().numpy())
+  gt = np.concatenate(gt)
+  del dd, score
+
+  nns = torch.empty((nq, k), dtype=torch.int32, device="cuda")
+  dist = torch.empty((nq, k), dtype=torch.float32, device="cuda")
+  found = torch.empty(nq, dtype=torch.int32, device="cuda")
+  stats = torch.zeros((nq, 4), dtype=torch.int32, device="cuda")
+  torch.cuda.synchronize()
+
+  def step(with_stats=False):
+    return eng.search_knn_device(qq.data_ptr(), nq, k, ef, nns.data_ptr(), dist.data_ptr(), found.data_ptr(),
+                                 stats.data_ptr() if with_stats else None)
+
+  step(with_stats=True)
+  st = stats.cpu().numpy().astype(np.int64)
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  kernel_ms = []
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    kernel_ms.append(step())             # synchronous: returns after the kernel finished
+  torch.cuda.synchronize()
+  elapsed = time.perf_counter() - t0
+  ids = nns.cpu().numpy()
+  recall = float(np.mean([len(set(a) & set(b)) / k for a, b in zip(ids, gt)]))
+
+  avg_kernel_ms = float(np.mean(kernel_ms))
+  gather_bytes = int(st[:, 0].sum()) * 4 * d
+  achieved = gather_bytes / (avg_kernel_ms * 1e-3) / 1e9
+  out = {
+      "metric": "batch search QPS at recall@%d (%s: %dx%d %s), with build seconds" % (
+          k, args.workload, n, d, "angular" if o["dist_type"] == "dot" else "l2"),
+      "value": nq * args.steps / elapsed,
+      "unit": "queries/s",
+      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+      "ms_per_step": elapsed / args.steps * 1e3,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "f32", "data": "synthetic",
+      "config": {"workload": "%s: %dx%d %s max_m=%d max_m0=%d ef_construction=%d; %d queries topk=%d ef_search=%d" % (
+          args.workload, n, d, o["dist_type"], o["max_m"], o["max_m0"], o["ef_construction"], nq, k, ef)},
+      "build_seconds": build_s,
+      "recall_at_k": recall,
+      "upload_seconds": upload_s, "datagen_seconds": gen_s,
+      "kernel_ms": avg_kernel_ms,
+      "per_query": {"n_dist": float(st[:, 0].mean()), "n_hops": float(st[:, 1].mean()),
+                    "n_dist_upper": float(st[:, 2].mean()), "n_sweeps_upper": float(st[:, 3].mean())},
+      "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
+                   "frac": achieved / 8000.0, "traffic": None,
+                   "kernel": "search_kernel", "algorithmic_bytes_per_launch": gather_bytes},
+  }
+
+  if not args.no_cpu:
+    from oracle import oracle as orc
+    cores = orc.host_threads()
+    idx_path = os.path.join(tmpdir, "bench.idx")
+    eng.save_index(idx_path)
+    ix = orc.OracleIndex(o["dist_type"]).load(idx_path)
+    os.remove(idx_path)
+    n_s = min(nq, 10000)
+    passes = 5
+    t0 = time.perf_counter()
+    for _ in range(passes):
+      o_ids, o_d, o_f = ix.search(queries[:n_s], k, ef, threads=cores)
+    cpu_search_s = (time.perf_counter() - t0) / passes
+    mism = int((o_ids != ids[:n_s]).any(axis=1).sum())
+    n_b = min(n, 400000)
+    t0 = time.perf_counter()
+    orc.OracleIndex(o["dist_type"]).build(data[:n_b], levels[:n_b], o["max_m"], o["max_m0"], o["ef_construction"],
+                                          mult, threads=cores)
+    cpu_build_s = time.perf_counter() - t0
+    out["cpu_baseline"] = {
+        "value": n_s / cpu_search_s, "unit": "queries/s", "cores": cores, "kind": "port",
+        "sample": "CPU oracle (hnswlib-semantics search) on the GPU-built index file, first %d queries x %d passes, "
+                  "topk=%d ef_search=%d; build sample: first %d points inserted in %.2f s (%.0f points/s)" % (
+                      n_s, passes, k, ef, n_b, cpu_build_s, n_b / cpu_build_s),
+        "build_points_per_s": n_b / cpu_build_s,
+        "gpu_build_points_per_s": n / build_s,
+    }
+    out["parity"] = {"queries_checked": n_s, "rows_with_id_mismatch_vs_oracle": mism}
+  print(json.dumps(out))
+
+
+if __name__ == "__main__":
+  main()

@@ -79,6 +79,11 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  // 1 = when a level is built, nodes that also live above are searched and re-selected
+  // again like the new ones (the reference processes every node of a level,
+  // cpp/include/cuda_build_kernels.cuh:188).  Off by default: replacing their rows
+  // drops reverse links they collected and measurably lowers recall on large sets.
+  int reprocess_upper = 0;
 
   // resident index
   int Dp = 0;
@@ -167,13 +172,14 @@ class Engine {
 
   void set_data(const float* data, int n, int d) {
     if (!data || n <= 0 || d <= 0) throw std::runtime_error("set_data: empty data");
-    need_device();
     host = HostIndex();
     host.N = n;
     host.D = d;
     host.vectors.assign(data, data + (size_t)n * d);
     have_levels = have_graph = host_links_stale = false;
-    upload_vectors();
+    pool_slots = 0;  // the slot pool is sized by N: rebuild it lazily
+    pool = SlotPool{};
+    if (has_device) upload_vectors();  // without a GPU only the host-side calls remain usable
     have_data = true;
   }
 
@@ -360,11 +366,19 @@ class Engine {
     std::vector<std::vector<int>> lists(host.maxlevel + 1);
     for (int i = 0; i < N; ++i)
       for (int l = 1; l <= host.levels[i]; ++l) lists[l].push_back(i);
-    std::vector<size_t> list_off(host.maxlevel + 2, 0);
+    std::vector<size_t> list_off(host.maxlevel + 2, 0), new_off(host.maxlevel + 2, 0);
+    std::vector<int> new_cnt(host.maxlevel + 2, 0);
     std::vector<int> flat;
     for (int l = 1; l <= host.maxlevel; ++l) {
       list_off[l] = flat.size();
       flat.insert(flat.end(), lists[l].begin(), lists[l].end());
+    }
+    for (int l = 0; l <= host.maxlevel; ++l) {
+      new_off[l] = flat.size();
+      if (!reprocess_upper)
+        for (int i = 0; i < N; ++i)
+          if (host.levels[i] == l) flat.push_back(i);
+      new_cnt[l] = (int)(flat.size() - new_off[l]);
     }
     d_level_nodes.reserve(std::max<size_t>(flat.size(), 1));
     if (!flat.empty()) HIP_CHECK(hipMemcpyAsync(d_level_nodes.p, flat.data(), flat.size() * 4, hipMemcpyHostToDevice, stream));
@@ -376,8 +390,12 @@ class Engine {
     const int glob_cap = std::max(4096, 8 * efc);
 
     for (int lv = host.maxlevel; lv >= 0; --lv) {
-      const int n_lv = lv == 0 ? N : (int)lists[lv].size();
+      int n_lv = lv == 0 ? N : (int)lists[lv].size();
       const int* nodes = lv == 0 ? nullptr : d_level_nodes.p + list_off[lv];
+      if (!reprocess_upper) {
+        n_lv = new_cnt[lv];
+        nodes = d_level_nodes.p + new_off[lv];
+      }
       const int S = lv == 0 ? host.S0 : host.SU;
       const int m_cap = lv == 0 ? host.max_m0 : host.max_m;
       int n_skel = 0;
@@ -577,6 +595,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "search_slots") e->impl.search_slots = (int)value;
   else if (n == "cand_lds") e->impl.cand_lds_override = (int)value;
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
+  else if (n == "reprocess_upper") e->impl.reprocess_upper = (int)value;
   else return -1;
   return 0;
 }

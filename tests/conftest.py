@@ -5,6 +5,14 @@ import sys
 import numpy as np
 import pytest
 
+# torch (used by GPU tests only to hold device buffers) ships its own copy of the HIP
+# runtime: it has to be loaded before libcuhnsw_amd.so pulls in the system one, or the
+# process ends up with two runtimes and torch finds no GPU.
+try:
+  import torch  # noqa: F401  pylint: disable=unused-import
+except ImportError:
+  torch = None
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
   sys.path.insert(0, ROOT)

@@ -1,0 +1,133 @@
+"""GPU build: graph invariants (checked by the oracle's validator on the saved file),
+recall against brute force compared with the CPU oracle's hnswlib-style build,
+determinism, and the Python API end to end."""
+import numpy as np
+import pytest
+
+from conftest import write_options
+from helpers import gauss_mixture, integer_vectors, recall
+
+pytestmark = pytest.mark.gpu
+
+
+def _build(tmp_path, x, levels, **opt):
+  from cuhnsw_amd import capi
+  e = capi.Engine()
+  path, full = write_options(tmp_path, **opt)
+  assert e.init(path) == 0
+  e.set_data(x)
+  e.set_random_levels(levels)
+  e.build_graph()
+  return e
+
+
+def _levels(n, mult, seed):
+  rng = np.random.default_rng(seed)
+  return (-np.log(np.maximum(rng.uniform(size=n), 1e-10)) * mult).astype(np.int32)
+
+
+CASES = [
+    ("dot50", 20000, 50, "dot", 12, 24, 110, "gauss"),
+    ("l2_128_int", 12000, 128, "l2", 16, 32, 100, "int"),
+    ("l2_960", 3000, 960, "l2", 16, 32, 60, "gauss_raw"),
+    ("dot96", 8000, 96, "dot", 16, 32, 80, "gauss"),
+]
+
+
+def _data(kind, n, d, seed):
+  if kind == "gauss":
+    return gauss_mixture(n, d, centres=200, seed=seed)
+  if kind == "gauss_raw":
+    return gauss_mixture(n, d, centres=100, seed=seed, normalise=False)
+  return integer_vectors(n, d, seed=seed, hi=219)
+
+
+@pytest.mark.parametrize("name,n,d,dist,max_m,max_m0,efc,kind", CASES, ids=[c[0] for c in CASES])
+def test_build_quality_and_invariants(oracle, tmp_path, name, n, d, dist, max_m, max_m0, efc, kind):
+  x = _data(kind, n, d, 21)
+  q = _data(kind, 300, d, 22)
+  mult = 1.0 / np.log(max_m)
+  levels = _levels(n, mult, 23)
+  e = _build(tmp_path, x, levels, dist_type=dist, max_m=max_m, max_m0=max_m0, ef_construction=efc,
+             heuristic_coef=0.0)
+  assert e.max_level == levels.max() and e.enter_point == int(np.argmax(levels))
+  p = str(tmp_path / "g.idx")
+  e.save_index(p)
+  ix = oracle.OracleIndex(dist).load(p)
+  assert ix.validate() == 0                       # ids in range, no self loops, no duplicates, degree caps, level membership
+  assert (ix.levels() == levels).all()
+  assert (ix.vectors() == x).all()
+  deg0 = ix.links0()[:, 0]
+  assert deg0.min() >= 1                          # nobody is left without links
+  gt, _ = oracle.bruteforce(x, q, 10, dist)
+  g_ids, g_d, g_f = e.search_knn(q, 10, 300)
+  # the file the GPU wrote, searched by the oracle: same answers
+  o_ids, o_d, o_f = ix.search(q, 10, 300)
+  assert (o_ids == g_ids).all() and (o_d == g_d).all() and (o_f == g_f).all()
+  r_gpu = recall(g_ids, gt)
+  cpu = oracle.OracleIndex(dist).build(x, levels, max_m, max_m0, efc, mult)
+  r_cpu = recall(cpu.search(q, 10, 300)[0], gt)
+  print("recall@10 gpu %.4f cpu %.4f mean deg0 %.2f" % (r_gpu, r_cpu, deg0.mean()))
+  assert r_gpu >= r_cpu - 0.005                   # within 0.5 points of the hnswlib-style CPU build
+  assert r_gpu >= 0.95
+
+
+def test_build_is_deterministic(tmp_path):
+  x = gauss_mixture(6000, 24, seed=31)
+  levels = _levels(6000, 0.4, 32)
+  files = []
+  for i in range(2):
+    e = _build(tmp_path, x, levels, max_m=8, max_m0=16, ef_construction=50)
+    p = str(tmp_path / ("d%d.idx" % i))
+    e.save_index(p)
+    files.append(open(p, "rb").read())
+  assert files[0] == files[1]
+
+
+def test_option_variants_keep_invariants(oracle, tmp_path):
+  x = gauss_mixture(5000, 16, seed=41)
+  levels = _levels(5000, 0.5, 42)
+  for opt in (dict(heuristic_coef=0.25), dict(save_remains=True), dict(heuristic_coef=0.5, save_remains=True)):
+    e = _build(tmp_path, x, levels, max_m=6, max_m0=12, ef_construction=40, **opt)
+    p = str(tmp_path / "v.idx")
+    e.save_index(p)
+    ix = oracle.OracleIndex("dot").load(p)
+    assert ix.validate() == 0
+    if opt.get("save_remains"):
+      assert ix.links0()[:, 0].mean() > 11.0      # pruned candidates fill the rows
+
+
+def test_tiny_builds(oracle, tmp_path):
+  for n in (1, 2, 3, 17):
+    x = gauss_mixture(n, 5, seed=n)
+    e = _build(tmp_path, x, _levels(n, 0.7, n), max_m=4, max_m0=8, ef_construction=10)
+    ids, d, f = e.search_knn(x, min(n, 3), 10)
+    assert (ids[:, 0] == np.arange(n)).all()     # every point finds itself
+    assert (f == min(n, 3)).all()
+
+
+def test_python_api_end_to_end(oracle, tmp_path):
+  from cuhnsw_amd import CuHNSW
+  x = gauss_mixture(10000, 50, centres=100, seed=51, normalise=False)
+  q = gauss_mixture(200, 50, centres=100, seed=52, normalise=True)
+  h = CuHNSW({"dist_type": "cosine", "nrz": True, "max_m": 12, "max_m0": 24, "ef_construction": 110,
+              "heuristic_coef": 0.0, "py_log_level": 1})
+  h.set_data(x)
+  np.testing.assert_allclose(np.linalg.norm(h.data, axis=1), 1.0, rtol=1e-5)
+  h.build()
+  nns, dist, found = h.search_knn(q, 10, 5)        # ef is raised to topk
+  assert nns.shape == (200, 10) and dist.dtype == np.float32 and (found == 10).all()
+  gt, _ = oracle.bruteforce(h.data, q, 10, "dot")
+  nns, dist, found = h.search_knn(q, 10, 300)
+  assert recall(nns, gt) >= 0.95
+  np.testing.assert_allclose(dist[:, 0], -(q * h.data[nns[:, 0]]).sum(1), rtol=1e-5, atol=1e-6)  # -dot convention
+  p = str(tmp_path / "api.idx")
+  h.save_index(p)
+  h2 = CuHNSW({"dist_type": "dot", "py_log_level": 1})
+  h2.load_index(p)
+  nns2, dist2, found2 = h2.search_knn(q, 10, 300)
+  assert (nns2 == nns).all() and (dist2 == dist).all()
+  one = h2.search_knn(q[0], 10, 300)              # 1-d query
+  assert (one[0][0] == nns[0]).all()
+  with pytest.raises(RuntimeError, match="dimension"):
+    h2.search_knn(np.zeros((2, 7), np.float32), 1, 1)

@@ -1,0 +1,177 @@
+"""GPU search parity: the HIP search (through the C ABI) against the CPU oracle on the
+same index file and queries — ids bit-exact, distances within 1e-5 relative (in fact
+bit-equal, both sides use the same canonical fp32 order), found counts and the
+per-query distance-evaluation / hop counters identical."""
+import numpy as np
+import pytest
+
+from conftest import write_options
+from helpers import gauss_mixture, integer_vectors, ring_graph
+
+pytestmark = pytest.mark.gpu
+
+
+def _engine(tmp_path, **opt):
+  from cuhnsw_amd import capi
+  e = capi.Engine()
+  path, _ = write_options(tmp_path, **opt)
+  assert e.init(path) == 0
+  return e
+
+
+def _levels(n, mult, seed):
+  rng = np.random.default_rng(seed)
+  return (-np.log(np.maximum(rng.uniform(size=n), 1e-10)) * mult).astype(np.int32)
+
+
+def _device_search(e, q, k, ef):
+  import torch
+  nq = q.shape[0]
+  qq = torch.from_numpy(np.ascontiguousarray(q, dtype=np.float32)).cuda()
+  nns = torch.empty((nq, k), dtype=torch.int32, device="cuda")
+  dist = torch.empty((nq, k), dtype=torch.float32, device="cuda")
+  found = torch.empty(nq, dtype=torch.int32, device="cuda")
+  stats = torch.zeros((nq, 4), dtype=torch.int32, device="cuda")
+  torch.cuda.synchronize()
+  e.search_knn_device(qq.data_ptr(), nq, k, ef, nns.data_ptr(), dist.data_ptr(), found.data_ptr(), stats.data_ptr())
+  return nns.cpu().numpy(), dist.cpu().numpy(), found.cpu().numpy(), stats.cpu().numpy()
+
+
+def _check_parity(oracle, ix, e, q, k, ef, counters=True):
+  o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
+  g_ids, g_d, g_f = e.search_knn(q, k, ef)
+  assert (g_f == o_f).all()
+  for r in range(q.shape[0]):
+    f = o_f[r]
+    assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d" % r
+    np.testing.assert_allclose(g_d[r, :f], o_d[r, :f], rtol=1e-5, atol=0)
+    assert (g_d[r, :f] == o_d[r, :f]).all()
+  if counters:
+    d_ids, d_d, d_f, stats = _device_search(e, q, k, ef)
+    assert (d_ids == g_ids).all() and (d_f == g_f).all()
+    assert (stats == o_cnt[:, :4]).all()
+
+
+CASES = [
+    # name, n, d, dist, max_m, max_m0, data kind
+    ("dot50", 6000, 50, "dot", 12, 24, "gauss"),        # one float4 per lane
+    ("dot96", 4000, 96, "dot", 16, 32, "gauss"),        # two
+    ("l2_128_int", 5000, 128, "l2", 16, 32, "int"),     # integer data: exact sums, many ties
+    ("l2_200", 3000, 200, "l2", 8, 16, "gauss_raw"),    # four
+    ("l2_960", 1500, 960, "l2", 16, 32, "gauss_raw"),   # query staged in LDS
+    ("dot7", 3000, 7, "dot", 5, 10, "gauss"),           # odd small dimension, odd degrees
+    ("l2_tiny_int", 4000, 6, "l2", 6, 12, "tiny_int"),  # almost everything ties
+]
+
+
+def _data(kind, n, d, seed):
+  if kind == "gauss":
+    return gauss_mixture(n, d, seed=seed)
+  if kind == "gauss_raw":
+    return gauss_mixture(n, d, seed=seed, normalise=False)
+  if kind == "int":
+    return integer_vectors(n, d, seed=seed, hi=219)
+  return integer_vectors(n, d, seed=seed, hi=4)
+
+
+@pytest.mark.parametrize("name,n,d,dist,max_m,max_m0,kind", CASES, ids=[c[0] for c in CASES])
+def test_search_parity_on_oracle_built_index(oracle, tmp_path, name, n, d, dist, max_m, max_m0, kind):
+  x = _data(kind, n, d, 1)
+  q = _data(kind, 200, d, 2)
+  mult = 1.0 / np.log(max_m)
+  ix = oracle.OracleIndex(dist).build(x, _levels(n, mult, 3), max_m, max_m0, 60, mult)
+  p = str(tmp_path / "i.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=max_m0)
+  e.load_index(p)
+  assert (e.num_data, e.num_dims, e.max_level, e.enter_point) == (n, d, ix.maxlevel, ix.enterpoint)
+  for k, ef in ((10, 300), (1, 1), (10, 10), (100, 64), (100, 120), (7, 33)):
+    _check_parity(oracle, ix, e, q, k, ef)
+
+
+def test_labels_from_file_are_returned(oracle, tmp_path):
+  n, d = 3000, 20
+  x = gauss_mixture(n, d, seed=4)
+  q = gauss_mixture(64, d, seed=5)
+  levels = _levels(n, 0.4, 6)
+  base = oracle.OracleIndex("dot").build(x, levels, 8, 16, 40, 0.4)
+  labels = np.random.default_rng(0).permutation(n).astype(np.uint64) * 3 + 5
+  l0 = base.links0()
+  up = np.concatenate([np.concatenate([[len(base.links(i, l))], np.pad(base.links(i, l), (0, 8 - len(base.links(i, l))))])
+                       for i in range(n) for l in range(1, levels[i] + 1)]).astype(np.uint32)
+  ix = oracle.OracleIndex("dot").from_arrays(x, levels, l0, up, 8, 16, base.maxlevel, base.enterpoint, labels=labels)
+  p = str(tmp_path / "lab.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="dot", max_m=8, max_m0=16)
+  e.load_index(p)
+  _check_parity(oracle, ix, e, q, 10, 50, counters=False)
+  g_ids, _, _ = e.search_knn(q, 10, 50)
+  assert set(np.unique(g_ids)) <= set(labels.astype(np.int64))
+
+
+def test_single_query_1d_and_tiny_indexes(oracle, tmp_path):
+  # N = 1
+  one = oracle.OracleIndex("l2").from_arrays(np.array([[1.0, 2.0]], np.float32), np.zeros(1, np.int32),
+                                             np.zeros((1, 5), np.uint32), np.zeros(0, np.uint32), 2, 4, 0, 0)
+  p = str(tmp_path / "one.idx")
+  one.save(p)
+  e = _engine(tmp_path, dist_type="l2", max_m=2, max_m0=4)
+  e.load_index(p)
+  ids, d, f = e.search_knn(np.array([0.0, 0.0], np.float32), 3, 10)  # 1-d query = one query
+  assert ids.shape == (1, 3) and f[0] == 1 and ids[0, 0] == 0 and d[0, 0] == 5.0
+  assert ids[0, 1] == -1 and np.isinf(d[0, 1])
+  # two components: found < topk
+  pts = np.arange(5, dtype=np.float32)[:, None]
+  links0 = np.zeros((5, 3), np.uint32)
+  links0[0] = [2, 1, 2]; links0[1] = [2, 0, 2]; links0[2] = [2, 0, 1]
+  links0[3] = [1, 4, 0]; links0[4] = [1, 3, 0]
+  ix = oracle.OracleIndex("l2").from_arrays(pts, np.zeros(5, np.int32), links0, np.zeros(0, np.uint32), 2, 2, 0, 0)
+  p = str(tmp_path / "comp.idx")
+  ix.save(p)
+  e.load_index(p)
+  ids, d, f = e.search_knn(np.array([[3.6]], np.float32), 5, 10)
+  assert f[0] == 3 and list(ids[0, :3]) == [2, 1, 0]
+  _check_parity(oracle, ix, e, np.array([[3.6], [0.2], [-5.0]], np.float32), 5, 10)
+
+
+def test_ef_ge_n_is_exact_brute_force(oracle, tmp_path):
+  n, d, k = 500, 12, 10
+  x = gauss_mixture(n, d, seed=8)
+  q = gauss_mixture(40, d, seed=9)
+  ix = oracle.OracleIndex("dot").from_arrays(x, np.zeros(n, np.int32), ring_graph(n, 8), np.zeros(0, np.uint32),
+                                             4, 8, 0, 0)
+  p = str(tmp_path / "ring.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="dot", max_m=4, max_m0=8)
+  e.load_index(p)
+  e.set_tunable("hnswlib_dist", 1)
+  ids, dists, found = e.search_knn(q, k, n)
+  bf_ids, bf_d = oracle.bruteforce(x, q, k, "dot")
+  assert (found == k).all() and (ids == bf_ids).all() and (dists == bf_d).all()
+
+
+def test_candidate_queue_spills_to_global_memory(oracle, tmp_path):
+  """A tiny LDS share for the candidate queue forces the global-memory overflow path;
+  results must not change."""
+  n, d = 8000, 32
+  x = gauss_mixture(n, d, seed=10)
+  q = gauss_mixture(100, d, seed=11)
+  mult = 1 / np.log(8)
+  ix = oracle.OracleIndex("dot").build(x, _levels(n, mult, 12), 8, 16, 60, mult)
+  p = str(tmp_path / "s.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="dot", max_m=8, max_m0=16)
+  e.load_index(p)
+  e.set_tunable("cand_lds", 64)
+  _check_parity(oracle, ix, e, q, 10, 400)
+  e.set_tunable("search_slots", 3)  # many queries per resident wavefront: visited sets must be clean between queries
+  _check_parity(oracle, ix, e, q, 10, 100)
+
+
+def test_errors(tmp_path):
+  e = _engine(tmp_path)
+  e.set_data(np.zeros((8, 4), np.float32))
+  with pytest.raises(RuntimeError, match="no index"):
+    e.search_knn(np.zeros((1, 4), np.float32), 1, 1)
+  with pytest.raises(RuntimeError, match="set_random_levels first"):
+    e.build_graph()
