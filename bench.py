@@ -38,6 +38,8 @@ def main():
   ap.add_argument("--n", type=int, default=None, help="shrink the data set (debugging)")
   ap.add_argument("--nq", type=int, default=None)
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--copy-calibration", action="store_true",
+                  help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     print("bench.py: this build runs on ONE GPU (the index and the query batch live on a single "
@@ -115,6 +117,14 @@ def main():
   elapsed = time.perf_counter() - t0
   ids = nns.cpu().numpy()
   recall = float(np.mean([len(set(a) & set(b)) / k for a, b in zip(ids, gt)]))
+
+  if args.copy_calibration:
+    src = torch.full((64 * 1024 * 1024,), 1.0, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+      dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
   avg_kernel_ms = float(np.mean(kernel_ms))
   gather_bytes = int(st[:, 0].sum()) * 4 * d
