@@ -8,7 +8,8 @@
 //     Replaces dot / squaresum / GetDistanceByVec of the reference
 //     (cpp/include/cuda_dist_kernels.cuh:13-124), which reduce over a 32-thread
 //     block through shared memory.
-//   * candidate queues live in LDS and reproduce libstdc++ heaps (heap_emul.h);
+//   * candidate queues live in LDS and reproduce libstdc++ heaps, each push / pop
+//     executed cooperatively by the wavefront (heap_coop.h);
 //     replaces the global-memory, thread-0 heap of the reference
 //     (cpp/include/cuda_heap_kernels.cuh:13-49) and its GetCand / CheckAlreadyExists
 //     scans (cpp/include/cuda_utils_kernels.cuh:50-151).
@@ -24,7 +25,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "heap_emul.h"
+#include "heap_coop.h"
 #include "index_file.h"
 #include "options.h"
 
@@ -161,6 +162,31 @@ __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const flo
   }
 }
 
+// one pass over 4*U rows starting at ids[r]: loads first, arithmetic after
+template <int DT, int R, int U, bool RAW>
+__device__ __forceinline__ void dist_pass(const float4* rows, int rowlen, const float4* q, const uint32_t* ids, int r, int n,
+                                          float* out, int g, int sub) {
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 v[U][R];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int idx = r + 4 * u + g;
+    const uint32_t id = ids[idx < n ? idx : n - 1];
+    const float4* p = rows + (size_t)id * rowlen + sub;
+#pragma unroll
+    for (int k = 0; k < R; ++k) v[u][k] = (sub + 16 * k < rowlen) ? p[16 * k] : zero;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
+#pragma unroll
+    for (int k = 0; k < R; ++k) acc4<DT>(q[k], v[u][k], ax, ay, az, aw);
+    const float key = finish16<DT, RAW>(ax, ay, az, aw);
+    const int idx = r + 4 * u + g;
+    if (sub == 0 && idx < n) out[idx] = key;
+  }
+}
+
 // keys of ids[0..n) (LDS) against the query -> out[0..n) (LDS).  n is wavefront-uniform.
 template <int DT, int QR, bool RAW>
 __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds,
@@ -168,31 +194,25 @@ __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv
   const int g = lane >> 4, sub = lane & 15;
   const int rowlen = ix.Dp >> 2;
   const float4* rows = reinterpret_cast<const float4*>(ix.vectors);
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   if (QR > 0) {
     constexpr int R = QR > 0 ? QR : 1;
-    constexpr int U = R == 1 ? 4 : (R == 2 ? 2 : 1);  // groups of 4 rows in flight
-    for (int r = 0; r < n; r += 4 * U) {
-      float4 v[U][R];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        int idx = r + 4 * u + g;
-        uint32_t id = ids[idx < n ? idx : n - 1];
-        const float4* p = rows + (size_t)id * rowlen + sub;
-#pragma unroll
-        for (int k = 0; k < R; ++k) v[u][k] = (sub + 16 * k < rowlen) ? p[16 * k] : zero;
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
-#pragma unroll
-        for (int k = 0; k < R; ++k) acc4<DT>(qv.q[k], v[u][k], ax, ay, az, aw);
-        float key = finish16<DT, RAW>(ax, ay, az, aw);
-        int idx = r + 4 * u + g;
-        if (sub == 0 && idx < n) out[idx] = key;
+    constexpr int UMAX = R == 1 ? 4 : (R == 2 ? 2 : 1);  // groups of 4 rows in flight
+    int r = 0;
+    while (r < n) {
+      const int rem = n - r;
+      if (UMAX >= 4 && rem > 8) {
+        dist_pass<DT, R, (UMAX >= 4 ? 4 : 1), RAW>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        r += 16;
+      } else if (UMAX >= 2 && rem > 4) {
+        dist_pass<DT, R, (UMAX >= 2 ? 2 : 1), RAW>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        r += 8;
+      } else {
+        dist_pass<DT, R, 1, RAW>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        r += 4;
       }
     }
   } else {
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     const int nk = (rowlen + 15) >> 4;
     for (int r = 0; r < n; r += 4) {
       int idx = r + g;
@@ -276,25 +296,26 @@ __device__ __forceinline__ void undo_visited(Scratch& s, SearchState& st, int la
 
 // Offers nbuf/dbuf[0..n) to the two queues in stored order (hnswlib's accept rule,
 // identical to the reference's, cpp/include/cuda_utils_kernels.cuh:220-225).
-// Executed by ONE lane.
-__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, int n, int ef) {
+// Wavefront-uniform: every lane runs it, the heap moves are cooperative.
+__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, int n, int ef, int lane) {
   LdsHeap top{s.top};
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
   for (int t = 0; t < n; ++t) {
-    float d = s.dbuf[t];
-    if (st.top_size < ef || st.lower > d) {
+    HeapEnt e;
+    e.key = s.dbuf[t];
+    e.id = s.nbuf[t];
+    e = uniform_ent(e);
+    if (st.top_size < ef || st.lower > e.key) {
       if (st.cand_size >= cand_cap) {
         st.fail = 1;
         return;
       }
-      HeapEnt e;
-      e.key = d;
-      e.id = s.nbuf[t];
-      heap_push<true>(cand, st.cand_size, e);
-      heap_push<false>(top, st.top_size, e);
-      if (st.top_size > ef) heap_pop<false>(top, st.top_size);
-      st.lower = s.top[0].key;
+      coop_push<true>(cand, st.cand_size, e, lane);
+      coop_push<false>(top, st.top_size, e, lane);
+      if (st.top_size > ef) coop_pop<false>(top, st.top_size, lane);
+      __syncthreads();
+      st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
     }
   }
 }
@@ -316,27 +337,22 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
     }
     __syncthreads();
     int cid = -1;
-    if (lane == 0) {
-      accept_list(s, st, n, ef);
-      if (!st.fail && st.cand_size > 0) {
-        HeapEnt c = cand.get(0);
-        bool stop = BUILD ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
-        if (!stop) {
-          cid = (int)c.id;
-          heap_pop<true>(cand, st.cand_size);
-        }
+    accept_list(s, st, n, ef, lane);
+    if (!st.fail && st.cand_size > 0) {
+      __syncthreads();
+      const HeapEnt c = uniform_ent(cand.get(0));
+      const bool stop = BUILD ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
+      if (!stop) {
+        cid = (int)c.id;
+        coop_pop<true>(cand, st.cand_size, lane);
       }
     }
-    cid = __builtin_amdgcn_readfirstlane(cid);
     __syncthreads();
     if (cid < 0) break;
     st.n_hops += 1;
     n = visit_row(link_row(ix, (uint32_t)cid, level), S, s, st, lane);
     __syncthreads();
   }
-  st.top_size = __builtin_amdgcn_readfirstlane(st.top_size);
-  st.cand_size = __builtin_amdgcn_readfirstlane(st.cand_size);
-  st.fail = __builtin_amdgcn_readfirstlane(st.fail);
 }
 
 // Greedy descent through levels from_level .. to_level+1 (hnswlib searchKnn upper

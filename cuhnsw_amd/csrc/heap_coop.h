@@ -1,0 +1,124 @@
+// Binary heaps that reproduce, move for move, what libstdc++'s
+// std::priority_queue<pair<float,unsigned>, vector<...>, CompareByFirst> does
+// (std::push_heap / std::pop_heap, bits/stl_heap.h: __push_heap, __adjust_heap),
+// executed cooperatively by the 64 lanes of one wavefront.
+//
+// Why literal: the search must return the ids hnswlib returns, and under equal
+// distances hnswlib's answer is a function of the heap's array layout.  Any other
+// priority-queue implementation is only equivalent while all keys are distinct.
+// (Replaces the thread-0 heap of the reference, cpp/include/cuda_heap_kernels.cuh:13-49.)
+//
+// Why cooperative: a sift is a chain of dependent LDS reads when one lane does it.
+// Here
+//   * sift-up (__push_heap): lane j reads the j-th ancestor of the hole, one ballot
+//     tells how far the value rises, one masked write shifts the ancestors down and
+//     drops the value — one LDS round trip whatever the depth;
+//   * sift-down (__adjust_heap): the hole's path always takes the child that is not
+//     "less", independent of the value, so 63 lanes evaluate that choice for every
+//     node of a 6-level subtree at once (one LDS round trip), the path is read off
+//     two ballot masks with scalar code, and the lanes on the path move their chosen
+//     child up.  Heaps up to 127 entries need one such stage, up to 8191 two.
+//
+// All functions must be called by all 64 lanes with wavefront-uniform arguments.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cuhnsw_amd {
+
+struct __attribute__((aligned(8))) HeapEnt {
+  float key;
+  uint32_t id;
+};
+
+// MINQ = false: max-queue on key (hnswlib top_candidates).
+// MINQ = true : hnswlib's candidate_set, a max-queue on (-key); comparing -a < -b is
+//               exactly a > b for non-NaN floats, so the key is stored unnegated.
+template <bool MINQ>
+__device__ __forceinline__ bool heap_less(float a, float b) {
+  return MINQ ? (a > b) : (a < b);
+}
+
+__device__ __forceinline__ HeapEnt uniform_ent(HeapEnt e) {
+  HeapEnt r;
+  r.key = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, e.key)));
+  r.id = (uint32_t)__builtin_amdgcn_readfirstlane((int)e.id);
+  return r;
+}
+
+// __push_heap(first, holeIndex = i, topIndex = 0, value = v)
+template <bool MINQ, class Acc>
+__device__ __forceinline__ void coop_sift_up(Acc& h, int i, HeapEnt v, int lane) {
+  __syncthreads();
+  const int q = lane < 31 ? ((i + 1) >> (lane + 1)) : 0;  // index + 1 of the (lane+1)-th ancestor
+  const bool valid = q >= 1;
+  HeapEnt e = v;
+  if (valid) e = h.get(q - 1);
+  const bool rises = valid && heap_less<MINQ>(e.key, v.key);
+  const unsigned long long m = __ballot(rises);
+  const int t = __builtin_ctzll(~m);  // ancestors passed on the way up
+  if (lane <= t) {
+    const int slot = ((i + 1) >> lane) - 1;
+    h.set(slot, lane < t ? e : v);
+  }
+}
+
+// priority_queue::emplace
+template <bool MINQ, class Acc>
+__device__ __forceinline__ void coop_push(Acc& h, int& size, HeapEnt v, int lane) {
+  coop_sift_up<MINQ>(h, size, v, lane);
+  size = size + 1;
+}
+
+// priority_queue::pop
+template <bool MINQ, class Acc>
+__device__ __forceinline__ void coop_pop(Acc& h, int& size, int lane) {
+  if (size > 1) {
+    __syncthreads();
+    const int len = size - 1;
+    const HeapEnt value = uniform_ent(h.get(len));
+    // lane t < 63 stands for the t-th node (breadth first) of the subtree under the hole
+    const int d = 31 - __clz(lane + 1);
+    const int o = lane + 1 - (1 << d);
+    int hole = 0;
+    for (;;) {
+      const int P = ((hole + 1) << d) - 1 + o;
+      const int c1 = 2 * P + 1;
+      const bool has1 = lane < 63 && c1 < len;
+      const bool has2 = lane < 63 && c1 + 1 < len;
+      HeapEnt L = value, R = value;
+      if (has1) {
+        L = h.get(c1);
+        R = h.get(c1 + 1);  // c1 + 1 <= len is a valid slot
+      }
+      const bool take_left = has1 && (!has2 || heap_less<MINQ>(R.key, L.key));
+      const unsigned long long mc = __ballot(has1);
+      const unsigned long long ml = __ballot(take_left);
+      unsigned long long path = 0ull;
+      int tt = 0, next = -1;
+#pragma unroll
+      for (int lvl = 0; lvl < 6; ++lvl) {
+        if (((mc >> tt) & 1ull) == 0ull) break;
+        path |= 1ull << tt;
+        const int ct = 2 * tt + 2 - (int)((ml >> tt) & 1ull);
+        if (ct >= 63) {
+          next = ((hole + 1) << 6) - 1 + (ct - 63);
+          break;
+        }
+        tt = ct;
+      }
+      if ((path >> lane) & 1ull) h.set(P, take_left ? L : R);
+      if (next < 0) {
+        const int dd = 31 - __clz(tt + 1);
+        hole = ((hole + 1) << dd) - 1 + (tt + 1 - (1 << dd));
+        break;
+      }
+      hole = next;
+      __syncthreads();
+    }
+    coop_sift_up<MINQ>(h, hole, value, lane);
+  }
+  size = size - 1;
+}
+
+}  // namespace cuhnsw_amd

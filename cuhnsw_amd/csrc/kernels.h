@@ -131,11 +131,11 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
 
     // keep the k best (literal pops), then order them by (key, label) ascending as
     // hnswlib's result queue does
-    if (lane == 0) {
+    {
       LdsHeap top{s.top};
-      while (st.top_size > a.k) heap_pop<false>(top, st.top_size);
+      while (st.top_size > a.k) coop_pop<false>(top, st.top_size, lane);
     }
-    const int T = __builtin_amdgcn_readfirstlane(st.top_size);
+    const int T = st.top_size;
     __syncthreads();
     uint64_t* tie = nullptr;
     if (ix.labels) {
