@@ -7,7 +7,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcuhnsw_amd.so")
+LIB_PATH = os.environ.get("CUHNSW_AMD_LIB") or os.path.join(_HERE, "libcuhnsw_amd.so")
 
 SYMBOLS = [
     "cuhnsw_create", "cuhnsw_destroy", "cuhnsw_last_error", "cuhnsw_init",

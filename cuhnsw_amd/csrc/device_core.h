@@ -57,10 +57,14 @@ struct Scratch {
   uint32_t* undo;      // global, ids whose bit is set
   int undo_cap;
   int bitmap_words;
+  HeapEnt* log;        // global, every accepted (key, id) in acceptance order
+  int log_cap;
+  StageTree tree;      // per-lane constants of the cooperative heap pop
 };
 
 struct SearchState {
-  int top_size, cand_size;
+  int top_size, cand_size;  // top_size: entries of the result set = min(accepted, ef)
+  int n_acc;                // accepted so far (= log entries)
   float lower;
   int undo_cnt;
   int n_dist, n_hops, n_dist_upper, n_sweeps;
@@ -294,11 +298,60 @@ __device__ __forceinline__ void undo_visited(Scratch& s, SearchState& st, int la
   st.undo_cnt = 0;
 }
 
-// Offers nbuf/dbuf[0..n) to the two queues in stored order (hnswlib's accept rule,
-// identical to the reference's, cpp/include/cuda_utils_kernels.cuh:220-225).
-// Wavefront-uniform: every lane runs it, the heap moves are cooperative.
-__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, int n, int ef, int lane) {
-  LdsHeap top{s.top};
+// The result set's KEYS, kept sorted in registers: lane L holds sorted positions
+// [L*NS, L*NS + NS).  hnswlib's search uses top_candidates only through its size and its
+// largest key (lowerBound), and both depend on the multiset of accepted keys alone, not on
+// the heap's layout — so during the search the ids are not needed and the eviction
+// "push, then pop the maximum" becomes one sorted insert (about 35 vector instructions, no
+// LDS).  Which ids survive is decided at the end from the log of accepted entries; only a
+// tie exactly at the k-th key needs the literal heap, which is then replayed from the log.
+// Unused positions hold +inf; when the set is full, evicted keys drift to positions >= ef,
+// where they are never read and never counted (they are >= the bound that admitted v).
+template <int NS>
+struct TopKeys {
+  float k[NS > 0 ? NS : 1];
+};
+template <int NS>
+__device__ __forceinline__ void topkeys_init(TopKeys<NS>& t) {
+#pragma unroll
+  for (int j = 0; j < (NS > 0 ? NS : 1); ++j) t.k[j] = INFINITY;
+}
+template <int NS>
+__device__ __forceinline__ void topkeys_insert(TopKeys<NS>& t, float v, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+  int c = 0;  // keys of this lane below v
+#pragma unroll
+  for (int j = 0; j < N; ++j) c += t.k[j] < v ? 1 : 0;
+  // previous lane's count and last key (lane 0: "all below", nothing to take over)
+  const int prev_c = __builtin_amdgcn_update_dpp(N, c, 0x138, 0xF, 0xF, false);  // wave_shr:1
+  const float prev_last = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t.k[N - 1]), 0x138, 0xF, 0xF, false));
+  const bool shifted = prev_c < N;         // the insertion happened in an earlier lane
+  const int pos = shifted ? 0 : c;         // c == N: this lane is untouched
+  const float incoming = shifted ? prev_last : v;
+#pragma unroll
+  for (int j = N - 1; j >= 0; --j) {
+    const float below = j > 0 ? t.k[j - 1] : incoming;
+    t.k[j] = j > pos ? below : (j == pos ? incoming : t.k[j]);
+  }
+}
+// key at sorted position pos (wavefront-uniform)
+template <int NS>
+__device__ __forceinline__ float topkeys_at(const TopKeys<NS>& t, int pos) {
+  constexpr int N = NS > 0 ? NS : 1;
+  const int l = pos / N, r = pos - l * N;
+  float x = t.k[0];
+#pragma unroll
+  for (int j = 1; j < N; ++j) x = r == j ? t.k[j] : x;
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l));
+}
+
+// Offers nbuf/dbuf[0..n) in stored order (hnswlib's accept rule, identical to the
+// reference's, cpp/include/cuda_utils_kernels.cuh:220-225).  Wavefront-uniform: every lane
+// runs it, the heap moves are cooperative.  NS > 0: result keys in registers (TopKeys);
+// NS == 0: literal result heap in LDS (s.top), for ef beyond the register capacity.
+template <int NS>
+__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys<NS>& tk, int n, int ef, int lane) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
   for (int t = 0; t < n; ++t) {
@@ -307,26 +360,43 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, int n, 
     e.id = s.nbuf[t];
     e = uniform_ent(e);
     if (st.top_size < ef || st.lower > e.key) {
-      if (st.cand_size >= cand_cap) {
+      if (st.cand_size >= cand_cap || (NS > 0 && st.n_acc >= s.log_cap)) {
         st.fail = 1;
         return;
       }
-      coop_push<true>(cand, st.cand_size, e, lane);
-      coop_push<false>(top, st.top_size, e, lane);
-      if (st.top_size > ef) coop_pop<false>(top, st.top_size, lane);
-      __syncthreads();
-      st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
+      if (NS > 0 && lane == 0) s.log[st.n_acc] = e;
+      st.n_acc += 1;
+      // the candidate queue normally fits its LDS share: keep that case on pure LDS
+      // instructions (the split accessor compiles to flat loads)
+      if (st.cand_size < s.cand_lds) {
+        LdsHeap cand_fast{s.cand};
+        coop_push<true>(cand_fast, st.cand_size, e, lane);
+      } else {
+        coop_push<true>(cand, st.cand_size, e, lane);
+      }
+      if (NS > 0) {
+        topkeys_insert<NS>(tk, e.key, lane);
+        st.top_size = st.n_acc < ef ? st.n_acc : ef;
+        st.lower = topkeys_at<NS>(tk, st.top_size - 1);
+      } else {
+        LdsHeap top{s.top};
+        coop_push<false>(top, st.top_size, e, lane);
+        if (st.top_size > ef) coop_pop<false>(top, st.top_size, s.tree, lane);
+        __syncthreads();
+        st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
+      }
     }
   }
 }
 
 // Best-first search of one level (hnswlib searchBaseLayerST / searchBaseLayer).
-// On entry s.nbuf[0..n_seed) holds seed ids that are already marked visited; on
-// exit s.top[0..st.top_size) is the result max-heap.  BUILD selects hnswlib's
+// On entry s.nbuf[0..n_seed) holds seed ids that are already marked visited.  On exit
+// the accepted entries are in s.log[0..st.n_acc) and tk holds the result keys (NS > 0), or
+// s.top[0..st.top_size) is the literal result max-heap (NS == 0).  BUILD selects hnswlib's
 // construction-time stop rule.
-template <int DT, int QR, bool BUILD>
+template <int DT, int QR, int NS, bool BUILD>
 __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
-                                             SearchState& st, int n_seed, int lane) {
+                                             SearchState& st, TopKeys<NS>& tk, int n_seed, int lane) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int S = row_stride(ix, level);
   int n = n_seed;
@@ -337,14 +407,19 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
     }
     __syncthreads();
     int cid = -1;
-    accept_list(s, st, n, ef, lane);
+    accept_list<NS>(s, st, tk, n, ef, lane);
     if (!st.fail && st.cand_size > 0) {
       __syncthreads();
-      const HeapEnt c = uniform_ent(cand.get(0));
+      const HeapEnt c = uniform_ent(s.cand[0]);
       const bool stop = BUILD ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
       if (!stop) {
         cid = (int)c.id;
-        coop_pop<true>(cand, st.cand_size, lane);
+        if (st.cand_size <= s.cand_lds) {
+          LdsHeap cand_fast{s.cand};
+          coop_pop<true>(cand_fast, st.cand_size, s.tree, lane);
+        } else {
+          coop_pop<true>(cand, st.cand_size, s.tree, lane);
+        }
       }
     }
     __syncthreads();
@@ -424,6 +499,46 @@ __device__ __forceinline__ void rank_sort(const HeapEnt* in, const uint64_t* tie
     out_id[rank] = me.id;
     out_key[rank] = me.key;
   }
+}
+
+// Collects from the log the entries that make up the k best: those with key <= bound.
+// Returns how many there are (they are stored while they fit cap).  More than `want`
+// means equal keys straddle the cut, which only the literal heap can resolve.
+__device__ __forceinline__ int collect_le(const HeapEnt* log, int n, float bound, HeapEnt* out, int cap, int lane) {
+  int cnt = 0;
+  for (int base = 0; base < n; base += 64) {
+    const int i = base + lane;
+    HeapEnt e;
+    e.key = INFINITY;
+    e.id = 0;
+    if (i < n) e = log[i];
+    const bool keep = i < n && e.key <= bound;
+    const unsigned long long mask = __ballot(keep);
+    const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+    if (keep && pos < cap) out[pos] = e;
+    cnt += __popcll(mask);
+  }
+  return cnt;
+}
+// Same with a strict bound first and ties filling up to `want` in log order (build: any
+// deterministic choice among equal keys is fine).
+__device__ __forceinline__ int collect_best(const HeapEnt* log, int n, float bound, int want, HeapEnt* out, int lane) {
+  int cnt = 0;
+  for (int pass = 0; pass < 2; ++pass) {
+    for (int base = 0; base < n && cnt < want; base += 64) {
+      const int i = base + lane;
+      HeapEnt e;
+      e.key = INFINITY;
+      e.id = 0;
+      if (i < n) e = log[i];
+      const bool keep = i < n && (pass == 0 ? e.key < bound : e.key == bound);
+      const unsigned long long mask = __ballot(keep);
+      const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+      if (keep && pos < want) out[pos] = e;
+      cnt += __popcll(mask);
+    }
+  }
+  return cnt < want ? cnt : want;
 }
 
 }  // namespace cuhnsw_amd

@@ -94,7 +94,7 @@ class Engine {
   DevBuf<int> d_levels;
   // per-wavefront slots
   DevBuf<uint32_t> d_bitmaps, d_undo;
-  DevBuf<HeapEnt> d_cand_glob;
+  DevBuf<HeapEnt> d_cand_glob, d_log;
   SlotPool pool{};
   int pool_slots = 0;
   DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count
@@ -224,18 +224,23 @@ class Engine {
   }
 
   // ---- slots -----------------------------------------------------------------------------
-  void ensure_pool(int slots, int cand_glob_cap) {
+  void ensure_pool(int slots, int cand_glob_cap, int log_cap) {
     const int words = (host.N + 31) / 32;
     const int undo_cap = std::min(32768, std::max(host.N, 64));
-    if (slots <= pool_slots && words == pool.bitmap_words && cand_glob_cap <= pool.cand_glob_cap && undo_cap == pool.undo_cap)
+    if (slots <= pool_slots && words == pool.bitmap_words && cand_glob_cap <= pool.cand_glob_cap &&
+        log_cap <= pool.log_cap && undo_cap == pool.undo_cap)
       return;
     slots = std::max(slots, pool_slots);
     cand_glob_cap = std::max(cand_glob_cap, pool.cand_glob_cap);
+    log_cap = std::max(log_cap, pool.log_cap);
     d_bitmaps.release();
     d_bitmaps.reserve((size_t)slots * words);
     HIP_CHECK(hipMemsetAsync(d_bitmaps.p, 0, (size_t)slots * words * 4, stream));
     d_undo.reserve((size_t)slots * undo_cap);
     d_cand_glob.reserve((size_t)slots * cand_glob_cap);
+    d_log.reserve((size_t)slots * log_cap);
+    pool.log = d_log.p;
+    pool.log_cap = log_cap;
     pool.bitmaps = d_bitmaps.p;
     pool.bitmap_words = words;
     pool.undo = d_undo.p;
@@ -249,8 +254,16 @@ class Engine {
     HIP_CHECK(hipMemsetAsync(d_bitmaps.p, 0, (size_t)pool_slots * pool.bitmap_words * 4, stream));
   }
 
-  int auto_cand_lds(int ef, int floor_entries, size_t fixed_bytes) const {
+  // slots of sorted result keys per lane: the result set lives in registers while
+  // ef < 64 * NS; 0 selects the literal LDS heap for larger ef
+  static int key_slots(int ef) { return ef < 320 ? 5 : (ef < 1024 ? 16 : 0); }
+
+  // LDS entries of the candidate queue.  With the result keys in registers the queue is the
+  // only large LDS user: 2*ef entries hold it in nearly every query (the rest spills to the
+  // slot's global area) and keep ~30 wavefronts per CU resident at ef = 300.
+  int auto_cand_lds(int ef, int ns, int floor_entries, size_t fixed_bytes) const {
     if (cand_lds_override > 0) return std::max(cand_lds_override, floor_entries);
+    if (ns > 0) return std::max(floor_entries, std::min(std::max(2 * ef, 128), 1024));
     const size_t budget = 10240;  // ~16 resident wavefronts per CU out of 160 KB LDS
     size_t used = fixed_bytes + (size_t)(ef + 1) * 8;
     int c = used < budget ? (int)((budget - used) / 8) : 0;
@@ -266,16 +279,16 @@ class Engine {
   }
 
   // ---- search ------------------------------------------------------------------------------
-  template <int DT, int QR>
+  template <int DT, int QR, int NS>
   void launch_search(const DevIndex& ix, SearchArgs& a, int max_slots_override, float* ms) {
-    const LdsPlan lp = plan_lds(QR, ix.Dp, a.ef, a.cand_lds, a.lcap, 0, 0);
-    auto kernel = search_kernel<DT, QR>;
+    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0);
+    auto kernel = search_kernel<DT, QR, NS>;
     int slots = resident_slots(kernel, lp.total);
     if (max_slots_override > 0) slots = max_slots_override;
     slots = std::max(1, std::min(slots, a.nq));
     int glob_cap = std::max(4096, 8 * a.ef);
     for (int attempt = 0; attempt < 6; ++attempt) {
-      ensure_pool(slots, glob_cap);
+      ensure_pool(slots, glob_cap, 2 * glob_cap);
       a.pool = pool;
       a.counter = d_ctl.p;
       a.status = d_ctl.p + 1;
@@ -290,9 +303,26 @@ class Engine {
       if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
       if (ctl[1] == 0) return;
       scrub_pool();
-      glob_cap *= 4;  // a candidate queue overflowed its global area: retry with more room
+      glob_cap *= 4;  // a candidate queue or accept log overflowed its global area: retry with more room
     }
     throw std::runtime_error("search: candidate queue overflow");
+  }
+  template <int DT, int QR>
+  void launch_search_ns(int ns, const DevIndex& ix, SearchArgs& a, float* ms) {
+    switch (ns) {
+      case 5: launch_search<DT, QR, 5>(ix, a, search_slots, ms); break;
+      case 16: launch_search<DT, QR, 16>(ix, a, search_slots, ms); break;
+      default: launch_search<DT, QR, 0>(ix, a, search_slots, ms); break;
+    }
+  }
+  template <int DT>
+  void launch_search_qr(int q, int ns, const DevIndex& ix, SearchArgs& a, float* ms) {
+    switch (q) {
+      case 1: launch_search_ns<DT, 1>(ns, ix, a, ms); break;
+      case 2: launch_search_ns<DT, 2>(ns, ix, a, ms); break;
+      case 4: launch_search_ns<DT, 4>(ns, ix, a, ms); break;
+      default: launch_search_ns<DT, 0>(ns, ix, a, ms); break;
+    }
   }
 
   void search_device(const float* d_qdata, int nq, int k, int ef, int* d_nns_out, float* d_dist_out, int* d_found_out,
@@ -310,16 +340,13 @@ class Engine {
     a.lcap = (std::max(std::max(host.S0, host.SU), std::max(k, 64)) + 63) / 64 * 64;
     const int q = qr();
     size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
-    a.cand_lds = auto_cand_lds(ef, std::max(k, 64), fixed);
-#define CUHNSW_DISPATCH_SEARCH(DT)                                             \
-  switch (q) {                                                                 \
-    case 1: launch_search<DT, 1>(ix, a, search_slots, ms); break;              \
-    case 2: launch_search<DT, 2>(ix, a, search_slots, ms); break;              \
-    case 4: launch_search<DT, 4>(ix, a, search_slots, ms); break;              \
-    default: launch_search<DT, 0>(ix, a, search_slots, ms); break;             \
-  }
-    if (dist_type == DIST_DOT) { CUHNSW_DISPATCH_SEARCH(DIST_DOT) } else { CUHNSW_DISPATCH_SEARCH(DIST_L2) }
-#undef CUHNSW_DISPATCH_SEARCH
+    const int ns = key_slots(ef);
+    // with the keys in registers the queue's LDS share doubles as result buffer (lcap entries,
+    // then lcap label slots) and as the replay heap (ef + 1 entries)
+    const int floor_entries = ns > 0 ? std::max(ef + 1, 2 * a.lcap) : std::max(k, 64);
+    a.cand_lds = auto_cand_lds(ef, ns, floor_entries, fixed);
+    if (dist_type == DIST_DOT) launch_search_qr<DIST_DOT>(q, ns, ix, a, ms);
+    else launch_search_qr<DIST_L2>(q, ns, ix, a, ms);
   }
 
   void search_host(const float* q, int nq, int k, int ef, int* nns, float* dists, int* found) {
@@ -340,7 +367,7 @@ class Engine {
   }
 
   // ---- build ---------------------------------------------------------------------------------
-  template <int DT, int QR>
+  template <int DT, int QR, int NS>
   void build_levels() {
     const int N = host.N;
     const int cap_in = 32;
@@ -384,7 +411,7 @@ class Engine {
     if (!flat.empty()) HIP_CHECK(hipMemcpyAsync(d_level_nodes.p, flat.data(), flat.size() * 4, hipMemcpyHostToDevice, stream));
 
     DevIndex ix = dev_index(d_dists0.p, d_distsU.p);
-    auto k_search = build_search_kernel<DT, QR>;
+    auto k_search = build_search_kernel<DT, QR, NS>;
     auto k_reverse = reverse_kernel<DT, QR>;
     const int efc = opt.ef_construction;
     const int glob_cap = std::max(4096, 8 * efc);
@@ -421,12 +448,12 @@ class Engine {
       const int q = QR;
       size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_cap * 8 + 64 +
                      (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
-      a.cand_lds = auto_cand_lds(efc, 64, fixed);
+      a.cand_lds = auto_cand_lds(efc, NS, 64, fixed);
       const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_cap);
       const LdsPlan lp3 = plan_lds(QR, Dp, S + cap_in, 0, a.lcap, S + cap_in, m_cap);
       const int slots1 = resident_slots(k_search, lp1.total);
       const int slots3 = resident_slots(k_reverse, lp3.total);
-      ensure_pool(slots1, glob_cap);
+      ensure_pool(slots1, glob_cap, 2 * glob_cap);
       a.pool = pool;
 
       int pos = 0;
@@ -457,6 +484,24 @@ class Engine {
     }
   }
 
+  template <int DT, int QR>
+  void build_ns(int ns) {
+    switch (ns) {
+      case 5: build_levels<DT, QR, 5>(); break;
+      case 16: build_levels<DT, QR, 16>(); break;
+      default: build_levels<DT, QR, 0>(); break;
+    }
+  }
+  template <int DT>
+  void build_qr(int q, int ns) {
+    switch (q) {
+      case 1: build_ns<DT, 1>(ns); break;
+      case 2: build_ns<DT, 2>(ns); break;
+      case 4: build_ns<DT, 4>(ns); break;
+      default: build_ns<DT, 0>(ns); break;
+    }
+  }
+
   void build_graph() {
     need_device();
     if (!have_data || !have_levels) throw std::runtime_error("build_graph: call set_data and set_random_levels first");
@@ -464,15 +509,9 @@ class Engine {
     HIP_CHECK(hipStreamSynchronize(stream));
     auto t0 = std::chrono::steady_clock::now();
     const int q = qr();
-#define CUHNSW_DISPATCH_BUILD(DT)               \
-  switch (q) {                                  \
-    case 1: build_levels<DT, 1>(); break;       \
-    case 2: build_levels<DT, 2>(); break;       \
-    case 4: build_levels<DT, 4>(); break;       \
-    default: build_levels<DT, 0>(); break;      \
-  }
-    if (dist_type == DIST_DOT) { CUHNSW_DISPATCH_BUILD(DIST_DOT) } else { CUHNSW_DISPATCH_BUILD(DIST_L2) }
-#undef CUHNSW_DISPATCH_BUILD
+    const int ns = key_slots(opt.ef_construction);
+    if (dist_type == DIST_DOT) build_qr<DIST_DOT>(q, ns);
+    else build_qr<DIST_L2>(q, ns);
     last_build_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     have_graph = true;
     host_links_stale = true;

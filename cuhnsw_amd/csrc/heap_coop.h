@@ -15,9 +15,10 @@
 //     drops the value — one LDS round trip whatever the depth;
 //   * sift-down (__adjust_heap): the hole's path always takes the child that is not
 //     "less", independent of the value, so 63 lanes evaluate that choice for every
-//     node of a 6-level subtree at once (one LDS round trip), the path is read off
-//     two ballot masks with scalar code, and the lanes on the path move their chosen
-//     child up.  Heaps up to 127 entries need one such stage, up to 8191 two.
+//     node of a 6-level subtree at once (one LDS round trip); a node is on the path if
+//     every edge from the subtree root down to it was the chosen one, which each lane
+//     tests against a ballot mask, and the lanes on the path move their chosen child
+//     up.  Heaps up to 127 entries need one such stage, up to 8191 two.
 //
 // All functions must be called by all 64 lanes with wavefront-uniform arguments.
 #pragma once
@@ -70,9 +71,29 @@ __device__ __forceinline__ void coop_push(Acc& h, int& size, HeapEnt v, int lane
   size = size + 1;
 }
 
+// per-lane constants of the 63-node stage tree used by coop_pop (lane t = t-th node in
+// breadth-first order): the parent's index and the set of edges from the stage root down
+// to the lane's node (bit x = edge into node x)
+struct StageTree {
+  int par;
+  unsigned long long anc;
+};
+__device__ __forceinline__ StageTree make_stage_tree(int lane) {
+  StageTree st;
+  st.par = lane >= 1 ? ((lane - 1) >> 1) : 0;
+  unsigned long long m = 0ull;
+  int x = lane < 63 ? lane : 0;
+  while (x > 0) {
+    m |= 1ull << x;
+    x = (x - 1) >> 1;
+  }
+  st.anc = m;
+  return st;
+}
+
 // priority_queue::pop
 template <bool MINQ, class Acc>
-__device__ __forceinline__ void coop_pop(Acc& h, int& size, int lane) {
+__device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tree, int lane) {
   if (size > 1) {
     __syncthreads();
     const int len = size - 1;
@@ -94,26 +115,23 @@ __device__ __forceinline__ void coop_pop(Acc& h, int& size, int lane) {
       const bool take_left = has1 && (!has2 || heap_less<MINQ>(R.key, L.key));
       const unsigned long long mc = __ballot(has1);
       const unsigned long long ml = __ballot(take_left);
-      unsigned long long path = 0ull;
-      int tt = 0, next = -1;
-#pragma unroll
-      for (int lvl = 0; lvl < 6; ++lvl) {
-        if (((mc >> tt) & 1ull) == 0ull) break;
-        path |= 1ull << tt;
-        const int ct = 2 * tt + 2 - (int)((ml >> tt) & 1ull);
-        if (ct >= 63) {
-          next = ((hole + 1) << 6) - 1 + (ct - 63);
-          break;
-        }
-        tt = ct;
-      }
-      if ((path >> lane) & 1ull) h.set(P, take_left ? L : R);
-      if (next < 0) {
-        const int dd = 31 - __clz(tt + 1);
-        hole = ((hole + 1) << dd) - 1 + (tt + 1 - (1 << dd));
+      // the edge parent -> this node is taken if the parent has children and chose this side
+      // (left children have odd indices); a node is on the hole's path if every edge from the
+      // stage root down to it is taken
+      const bool edge = lane >= 1 && lane < 63 && ((mc >> tree.par) & 1ull) != 0ull &&
+                        (int)((ml >> tree.par) & 1ull) == (lane & 1);
+      const unsigned long long me = __ballot(edge);
+      const bool on_path = lane < 63 && (me & tree.anc) == tree.anc;
+      const unsigned long long mp = __ballot(on_path);
+      if (on_path && has1) h.set(P, take_left ? L : R);
+      const int last = 63 - __builtin_clzll(mp);  // deepest node of the path inside this stage
+      const int dd = 31 - __clz(last + 1);
+      const int last_abs = ((hole + 1) << dd) - 1 + (last + 1 - (1 << dd));
+      if (((mc >> last) & 1ull) == 0ull) {
+        hole = last_abs;  // no child: the hole stops here
         break;
       }
-      hole = next;
+      hole = 2 * last_abs + 2 - (int)((ml >> last) & 1ull);  // its chosen child roots the next stage
       __syncthreads();
     }
     coop_sift_up<MINQ>(h, hole, value, lane);

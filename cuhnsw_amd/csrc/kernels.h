@@ -29,6 +29,8 @@ struct SlotPool {
   int undo_cap;
   HeapEnt* cand_glob;
   int cand_glob_cap;
+  HeapEnt* log;  // accepted entries of the running search
+  int log_cap;
 };
 
 struct SearchArgs {
@@ -93,13 +95,16 @@ __device__ __forceinline__ void bind_slot(Scratch& s, const SlotPool& pool, int 
   s.undo_cap = pool.undo_cap;
   s.cand_glob = pool.cand_glob + (size_t)slot * pool.cand_glob_cap;
   s.cand_glob_cap = pool.cand_glob_cap;
+  s.log = pool.log + (size_t)slot * pool.log_cap;
+  s.log_cap = pool.log_cap;
 }
 
-template <int DT, int QR>
+// NS > 0: result keys in registers (ef < 64*NS); NS == 0: literal result heap in LDS.
+template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, a.ef, a.cand_lds, a.lcap, 0, 0);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0);
   Scratch s;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
@@ -107,7 +112,11 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   s.cand_lds = a.cand_lds;
   s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
   s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
+  s.tree = make_stage_tree(lane);
   bind_slot(s, a.pool, blockIdx.x);
+  // after the search the candidate queue is dead: its LDS share (>= ef + 1 entries) then
+  // holds the collected results, or the literal heap when a tie has to be replayed
+  if (NS > 0) s.top = s.cand;
 
   for (;;) {
     int qi = 0;
@@ -117,8 +126,10 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     QVec<QR> qv;
     load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
     SearchState st;
-    st.top_size = 0; st.cand_size = 0; st.lower = 0.f; st.undo_cnt = 0;
+    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.undo_cnt = 0;
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
+    TopKeys<NS> tk;
+    topkeys_init<NS>(tk);
 
     uint32_t cur = ix.enterpoint;
     float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
@@ -127,19 +138,40 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     visit_single(s, st, cur, lane);
     if (lane == 0) s.nbuf[0] = cur;
     __syncthreads();
-    search_level<DT, QR, false>(ix, qv, 0, a.ef, s, st, 1, lane);
+    search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
 
-    // keep the k best (literal pops), then order them by (key, label) ascending as
-    // hnswlib's result queue does
-    {
-      LdsHeap top{s.top};
-      while (st.top_size > a.k) coop_pop<false>(top, st.top_size, lane);
+    // the k best.  With the keys in registers: the entries of the log at or below the k-th
+    // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the
+    // literal heap decides: replay every accepted entry through it, pop down to k.
+    int T = st.top_size < a.k ? st.top_size : a.k;
+    bool literal = NS == 0;
+    if (NS > 0 && !st.fail) {
+      __threadfence_block();
+      const float bound = topkeys_at<NS>(tk, T - 1);
+      const int cnt = collect_le(s.log, st.n_acc, bound, s.top, a.lcap, lane);
+      if (cnt != T) {
+        literal = true;
+        LdsHeap top{s.top};
+        int size = 0;
+        for (int i = 0; i < st.n_acc; ++i) {
+          const HeapEnt e = uniform_ent(s.log[i]);
+          coop_push<false>(top, size, e, lane);
+          if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
+        }
+        st.top_size = size;
+      }
     }
-    const int T = st.top_size;
+    if (literal) {
+      LdsHeap top{s.top};
+      while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
+      T = st.top_size;
+    }
     __syncthreads();
     uint64_t* tie = nullptr;
     if (ix.labels) {
-      tie = reinterpret_cast<uint64_t*>(s.cand);
+      // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
+      // whose first lcap entries hold the survivors themselves
+      tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
       for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
       __syncthreads();
     }
@@ -233,7 +265,7 @@ __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32
 }
 
 // Phase 1 of a build batch: search + select, read-only on the graph.
-template <int DT, int QR>
+template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
@@ -249,6 +281,7 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
   float* skey = reinterpret_cast<float*>(smem + lp.sorted_key);
   uint32_t* oid = reinterpret_cast<uint32_t*>(smem + lp.out_id);
   float* okey = reinterpret_cast<float*>(smem + lp.out_key);
+  s.tree = make_stage_tree(lane);
   bind_slot(s, a.pool, blockIdx.x);
 
   for (;;) {
@@ -260,8 +293,10 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     QVec<QR> qv;
     load_node_query<QR>(qv, s.qlds, ix, x, lane);
     SearchState st;
-    st.top_size = 0; st.cand_size = 0; st.lower = 0.f; st.undo_cnt = 0;
+    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.undo_cnt = 0;
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
+    TopKeys<NS> tk;
+    topkeys_init<NS>(tk);
     visit_single(s, st, x, lane);  // a node never links to itself
 
     int n_seed = 0;
@@ -286,9 +321,15 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
       n_seed = visit_row(link_row(ix, x, a.level), row_stride(ix, a.level), s, st, lane);
     }
     __syncthreads();
-    search_level<DT, QR, true>(ix, qv, a.level, a.efc, s, st, n_seed, lane);
+    search_level<DT, QR, NS, true>(ix, qv, a.level, a.efc, s, st, tk, n_seed, lane);
 
-    const int T = st.top_size;
+    // the efc best accepted entries (any deterministic choice among equal keys at the cut)
+    int T = st.top_size;
+    if (NS > 0 && T > 0) {
+      __threadfence_block();
+      T = collect_best(s.log, st.n_acc, topkeys_at<NS>(tk, T - 1), T, s.top, lane);
+    }
+    __syncthreads();
     rank_sort(s.top, nullptr, T, sid, skey, lane);
     __syncthreads();
     const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);

@@ -16,6 +16,7 @@ __global__ void __launch_bounds__(64) replay_kernel(const float* keys, int n_ops
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
   SplitHeap h{reinterpret_cast<HeapEnt*>(smem), glob, lds_cap};
+  const StageTree tree = make_stage_tree(lane);
   int size = 0;
   for (int op = 0; op < n_ops; ++op) {
     const float k = keys[op];
@@ -29,7 +30,7 @@ __global__ void __launch_bounds__(64) replay_kernel(const float* keys, int n_ops
       __syncthreads();
       HeapEnt root = uniform_ent(h.get(0));
       if (lane == 0) popped[op] = (int)root.id;
-      coop_pop<MINQ>(h, size, lane);
+      coop_pop<MINQ>(h, size, tree, lane);
     }
     if ((op + 1) % dump_every == 0) {
       __syncthreads();

@@ -83,22 +83,23 @@ def pop_coop(a, size, minq=False):
         if has1[lane]:
           left[lane], right[lane] = a[c1], a[c1 + 1]
         take_left[lane] = has1[lane] and ((not has2) or less(minq, right[lane][0], left[lane][0]))
-      tt, path, nxt = 0, [], None
-      for _ in range(6):
-        if not has1[tt]:
-          break
-        path.append(tt)
-        ct = 2 * tt + 2 - (1 if take_left[tt] else 0)
-        if ct >= 63:
-          nxt = ((hole + 1) << 6) - 1 + (ct - 63)
-          break
-        tt = ct
-      writes = [(pos[t], left[t] if take_left[t] else right[t]) for t in path]
+      # a node is on the hole's path iff every edge from the stage root down to it is the
+      # chosen one (the kernels test this against one ballot mask per lane)
+      def on_path(t):
+        while t > 0:
+          par = (t - 1) >> 1
+          if not has1[par] or take_left[par] != (t % 2 == 1):
+            return False
+          t = par
+        return True
+      path = [t for t in range(63) if on_path(t)]
+      writes = [(pos[t], left[t] if take_left[t] else right[t]) for t in path if has1[t]]
       for slot, e in writes:
         a[slot] = e
-      if nxt is None:
-        hole = pos[tt]
+      last = max(path)
+      if not has1[last]:
+        hole = pos[last]
         break
-      hole = nxt
+      hole = 2 * pos[last] + 2 - (1 if take_left[last] else 0)
     _sift_up_coop(a, hole, value, minq)
   return size - 1
