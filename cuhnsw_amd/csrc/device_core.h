@@ -162,7 +162,7 @@ __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const flo
       t.w = i + 3 < D ? src[i + 3] : 0.0f;
       qlds[c] = t;
     }
-    __syncthreads();
+    wave_sync();
   }
 }
 
@@ -354,12 +354,21 @@ template <int NS>
 __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys<NS>& tk, int n, int ef, int lane) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
-  for (int t = 0; t < n; ++t) {
-    HeapEnt e;
-    e.key = s.dbuf[t];
-    e.id = s.nbuf[t];
-    e = uniform_ent(e);
-    if (st.top_size < ef || st.lower > e.key) {
+  for (int base = 0; base < n; base += 64) {
+    // every lane takes one offer; offers that already fail against the current bound can
+    // be dropped at once (the bound never rises once the set is full), the others are
+    // taken in stored order and re-checked against the bound as it moves
+    const int mine = base + lane;
+    const float my_key = mine < n ? s.dbuf[mine] : INFINITY;
+    const uint32_t my_id = mine < n ? s.nbuf[mine] : 0u;
+    unsigned long long todo = __ballot(mine < n && (st.top_size < ef || st.lower > my_key));
+    while (todo != 0ull) {
+      const int j = __builtin_ctzll(todo);
+      todo &= todo - 1ull;
+      HeapEnt e;
+      e.key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+      e.id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+      if (!(st.top_size < ef || st.lower > e.key)) continue;
       if (st.cand_size >= cand_cap || (NS > 0 && st.n_acc >= s.log_cap)) {
         st.fail = 1;
         return;
@@ -382,7 +391,7 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
         LdsHeap top{s.top};
         coop_push<false>(top, st.top_size, e, lane);
         if (st.top_size > ef) coop_pop<false>(top, st.top_size, s.tree, lane);
-        __syncthreads();
+        wave_sync();
         st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
       }
     }
@@ -405,11 +414,11 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
       dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
       st.n_dist += n;
     }
-    __syncthreads();
+    wave_sync();
     int cid = -1;
     accept_list<NS>(s, st, tk, n, ef, lane);
     if (!st.fail && st.cand_size > 0) {
-      __syncthreads();
+      wave_sync();
       const HeapEnt c = uniform_ent(s.cand[0]);
       const bool stop = BUILD ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
       if (!stop) {
@@ -422,11 +431,11 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
         }
       }
     }
-    __syncthreads();
+    wave_sync();
     if (cid < 0) break;
     st.n_hops += 1;
     n = visit_row(link_row(ix, (uint32_t)cid, level), S, s, st, lane);
-    __syncthreads();
+    wave_sync();
   }
 }
 
@@ -443,12 +452,12 @@ __device__ __forceinline__ void descend(const DevIndex& ix, const QVec<QR>& qv, 
     while (changed) {
       changed = false;
       int n = load_row(link_row(ix, cur, level), ix.SU, s, lane);
-      __syncthreads();
+      wave_sync();
       st.n_sweeps += 1;
       if (n == 0) break;
       dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
       st.n_dist_upper += n;
-      __syncthreads();
+      wave_sync();
       float best = INFINITY;
       int bidx = -1;
       for (int base = 0; base < n; base += 64) {
@@ -466,7 +475,7 @@ __device__ __forceinline__ void descend(const DevIndex& ix, const QVec<QR>& qv, 
         cur = s.nbuf[bidx];
         changed = true;
       }
-      __syncthreads();
+      wave_sync();
     }
   }
 }
@@ -475,11 +484,11 @@ __device__ __forceinline__ void descend(const DevIndex& ix, const QVec<QR>& qv, 
 template <int DT, int QR>
 __device__ __forceinline__ float dist_single(const DevIndex& ix, const QVec<QR>& qv, uint32_t id, Scratch& s, int lane) {
   if (lane == 0) s.nbuf[0] = id;
-  __syncthreads();
+  wave_sync();
   dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, 1, s.dbuf, lane);
-  __syncthreads();
+  wave_sync();
   float d = s.dbuf[0];
-  __syncthreads();
+  wave_sync();
   return d;
 }
 

@@ -27,6 +27,16 @@
 
 namespace cuhnsw_amd {
 
+// Every kernel here runs one wavefront per workgroup, and a wavefront's LDS (and global)
+// instructions execute in program order, so lanes exchange data through memory without
+// waiting: what is needed between a write by one lane and a read by another is only that
+// the compiler keeps their order.  (__syncthreads() would also drain every outstanding
+// global access — a full memory round trip per call.)
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
 struct __attribute__((aligned(8))) HeapEnt {
   float key;
   uint32_t id;
@@ -50,7 +60,7 @@ __device__ __forceinline__ HeapEnt uniform_ent(HeapEnt e) {
 // __push_heap(first, holeIndex = i, topIndex = 0, value = v)
 template <bool MINQ, class Acc>
 __device__ __forceinline__ void coop_sift_up(Acc& h, int i, HeapEnt v, int lane) {
-  __syncthreads();
+  wave_sync();
   const int q = lane < 31 ? ((i + 1) >> (lane + 1)) : 0;  // index + 1 of the (lane+1)-th ancestor
   const bool valid = q >= 1;
   HeapEnt e = v;
@@ -95,7 +105,7 @@ __device__ __forceinline__ StageTree make_stage_tree(int lane) {
 template <bool MINQ, class Acc>
 __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tree, int lane) {
   if (size > 1) {
-    __syncthreads();
+    wave_sync();
     const int len = size - 1;
     const HeapEnt value = uniform_ent(h.get(len));
     // lane t < 63 stands for the t-th node (breadth first) of the subtree under the hole
@@ -132,7 +142,7 @@ __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tre
         break;
       }
       hole = 2 * last_abs + 2 - (int)((ml >> last) & 1ull);  // its chosen child roots the next stage
-      __syncthreads();
+      wave_sync();
     }
     coop_sift_up<MINQ>(h, hole, value, lane);
   }

@@ -137,7 +137,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
 
     visit_single(s, st, cur, lane);
     if (lane == 0) s.nbuf[0] = cur;
-    __syncthreads();
+    wave_sync();
     search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
 
     // the k best.  With the keys in registers: the entries of the log at or below the k-th
@@ -166,20 +166,20 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
       while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
       T = st.top_size;
     }
-    __syncthreads();
+    wave_sync();
     uint64_t* tie = nullptr;
     if (ix.labels) {
       // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
       // whose first lcap entries hold the survivors themselves
       tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
       for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
-      __syncthreads();
+      wave_sync();
     }
     rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
-    __syncthreads();
+    wave_sync();
     if (!a.hnswlib_dist && T > 0) {
       dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
-      __syncthreads();
+      wave_sync();
     }
     for (int r = lane; r < a.k; r += 64) {
       int out_id = -1;
@@ -203,7 +203,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
       }
     }
     undo_visited(s, st, lane);
-    __syncthreads();
+    wave_sync();
   }
 }
 
@@ -219,9 +219,9 @@ __device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, cons
     for (int k = 0; k < (QR > 0 ? QR : 1); ++k) qv.q[k] = (sub + 16 * k < rowlen) ? p[sub + 16 * k] : zero;
   } else {
     const int chunks = (rowlen + 15) / 16 * 16;
-    __syncthreads();
+    wave_sync();
     for (int c = lane; c < chunks; c += 64) qlds[c] = c < rowlen ? p[c] : zero;
-    __syncthreads();
+    wave_sync();
   }
 }
 
@@ -246,11 +246,11 @@ __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32
       QVec<QR> cv;
       load_node_query<QR>(cv, s.qlds, ix, c, lane);
       dist_list<DT, QR, false>(ix, cv, s.qlds, oid, head, s.dbuf, lane);
-      __syncthreads();
+      wave_sync();
       bool mine = false;
       for (int t = lane; t < head; t += 64) mine = mine || (dq > s.dbuf[t]);
       skip = __ballot(mine) != 0ull;
-      __syncthreads();
+      wave_sync();
     }
     if (!skip) {
       if (lane == 0) { oid[head] = c; okey[head] = dq; }
@@ -259,7 +259,7 @@ __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32
       if (lane == 0) { oid[tail] = c; okey[tail] = dq; }
       tail--;
     }
-    __syncthreads();
+    wave_sync();
   }
   return save_remains ? max_head : head;
 }
@@ -320,7 +320,7 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
       // x also lives above: start from the links it inherited at this level
       n_seed = visit_row(link_row(ix, x, a.level), row_stride(ix, a.level), s, st, lane);
     }
-    __syncthreads();
+    wave_sync();
     search_level<DT, QR, NS, true>(ix, qv, a.level, a.efc, s, st, tk, n_seed, lane);
 
     // the efc best accepted entries (any deterministic choice among equal keys at the cut)
@@ -329,9 +329,9 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
       __threadfence_block();
       T = collect_best(s.log, st.n_acc, topkeys_at<NS>(tk, T - 1), T, s.top, lane);
     }
-    __syncthreads();
+    wave_sync();
     rank_sort(s.top, nullptr, T, sid, skey, lane);
-    __syncthreads();
+    wave_sync();
     const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);
     for (int j = lane; j < a.m_cap; j += 64) {
       a.sel_ids[(size_t)b * a.m_cap + j] = j < deg ? oid[j] : kEmpty;
@@ -342,7 +342,7 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
       if (st.fail) *a.status = 1;
     }
     undo_visited(s, st, lane);
-    __syncthreads();
+    wave_sync();
   }
 }
 
@@ -413,7 +413,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       if (valid) { cbuf[pos].key = key; cbuf[pos].id = id; }
       n0 += __popcll(mask);
     }
-    __syncthreads();
+    wave_sync();
     // newcomers that are not linked yet
     int T = n0;
     for (int base = 0; base < nin; base += 64) {
@@ -430,20 +430,20 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       if (keep) cbuf[pos] = e;
       T += __popcll(mask);
     }
-    __syncthreads();
+    wave_sync();
     const int n_new = T - n0;
     if (n_new > 0) {
       if (T <= a.m_cap) {
         // room for all: append the newcomers, ordered by (key, id)
         rank_sort(cbuf + n0, nullptr, n_new, sid, skey, lane);
-        __syncthreads();
+        wave_sync();
         for (int t = lane; t < n_new; t += 64) {
           row[n0 + t] = sid[t];
           drow[n0 + t] = skey[t];
         }
       } else {
         rank_sort(cbuf, nullptr, T, sid, skey, lane);
-        __syncthreads();
+        wave_sync();
         const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);
         for (int j = lane; j < a.m_cap; j += 64) {
           row[j] = j < deg ? oid[j] : kEmpty;
@@ -452,7 +452,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       }
     }
     if (lane == 0) a.inbox_cnt[y] = 0;
-    __syncthreads();
+    wave_sync();
   }
 }
 

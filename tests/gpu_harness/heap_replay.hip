@@ -27,13 +27,13 @@ __global__ void __launch_bounds__(64) replay_kernel(const float* keys, int n_ops
       coop_push<MINQ>(h, size, e, lane);
       if (lane == 0) popped[op] = -1;
     } else {
-      __syncthreads();
+      wave_sync();
       HeapEnt root = uniform_ent(h.get(0));
       if (lane == 0) popped[op] = (int)root.id;
       coop_pop<MINQ>(h, size, tree, lane);
     }
     if ((op + 1) % dump_every == 0) {
-      __syncthreads();
+      wave_sync();
       HeapEnt* d = dumps + (size_t)(op / dump_every) * cap;
       for (int i = lane; i < size; i += 64) d[i] = h.get(i);
       if (lane == 0) sizes[op / dump_every] = size;
