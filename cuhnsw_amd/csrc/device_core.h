@@ -65,6 +65,7 @@ struct Scratch {
 struct SearchState {
   int top_size, cand_size;  // top_size: entries of the result set = min(accepted, ef)
   int n_acc;                // accepted so far (= log entries)
+  float maxkey;             // largest accepted key
   float lower;
   int undo_cnt;
   int n_dist, n_hops, n_dist_upper, n_sweeps;
@@ -80,9 +81,23 @@ struct SplitHeap {
   HeapEnt* lds;
   HeapEnt* glob;
   int nlds;
-  __device__ __forceinline__ HeapEnt get(int i) const { return i < nlds ? lds[i] : glob[i - nlds]; }
+  // The global branch waits for its own load at once (s_waitcnt vmcnt(0)).  It is the rare
+  // path; without the explicit wait the compiler merges both branches into one flat load
+  // and then has to drain ALL outstanding vector-memory traffic (the fire-and-forget log and
+  // undo stores too) before unrelated instructions of the hot loop.
+  __device__ __forceinline__ HeapEnt get(int i) const {
+    if (i < nlds) return lds[i];
+    HeapEnt r = glob[i - nlds];
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    return r;
+  }
   __device__ __forceinline__ void set(int i, HeapEnt e) {
-    if (i < nlds) lds[i] = e; else glob[i - nlds] = e;
+    if (i < nlds) {
+      lds[i] = e;
+    } else {
+      glob[i - nlds] = e;
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
   }
 };
 
@@ -216,19 +231,30 @@ __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv
       }
     }
   } else {
+    // long rows: 16 lanes still own one row (the summation order is tied to 16 lanes), so
+    // a lane has rowlen/16 chunks to fetch; they are issued eight at a time to keep eight
+    // 16-byte loads per lane in flight, the query chunks come from LDS
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     const int nk = (rowlen + 15) >> 4;
+    constexpr int B = 8;
     for (int r = 0; r < n; r += 4) {
-      int idx = r + g;
-      uint32_t id = ids[idx < n ? idx : n - 1];
+      const int idx = r + g;
+      const uint32_t id = ids[idx < n ? idx : n - 1];
       const float4* p = rows + (size_t)id * rowlen + sub;
       float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
-#pragma unroll 4
-      for (int k = 0; k < nk; ++k) {
-        float4 v = (sub + 16 * k < rowlen) ? p[16 * k] : zero;
-        acc4<DT>(qlds[sub + 16 * k], v, ax, ay, az, aw);
+      for (int k0 = 0; k0 < nk; k0 += B) {
+        float4 v[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) v[b] = (sub + 16 * (k0 + b) < rowlen) ? p[16 * (k0 + b)] : zero;
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          // chunks past the row end multiply zeros (the LDS copy is padded to a multiple of 16
+          // chunks, so only indices below that are read)
+          const float4 qq = (k0 + b < nk) ? qlds[sub + 16 * (k0 + b)] : zero;
+          acc4<DT>(qq, v[b], ax, ay, az, aw);
+        }
       }
-      float key = finish16<DT, RAW>(ax, ay, az, aw);
+      const float key = finish16<DT, RAW>(ax, ay, az, aw);
       if (sub == 0 && idx < n) out[idx] = key;
     }
   }
@@ -239,10 +265,18 @@ __device__ __forceinline__ const uint32_t* link_row(const DevIndex& ix, uint32_t
 }
 __device__ __forceinline__ int row_stride(const DevIndex& ix, int level) { return level == 0 ? ix.S0 : ix.SU; }
 
+// The visited bitmap of a slot is touched by one wavefront only; the atomic is there because
+// two lanes of that wavefront may hit the same word.  Workgroup scope is therefore enough
+// and lets the read-modify-write complete in the XCD's own L2 instead of being pushed out
+// to device-coherent memory as an agent-scope atomic (atomicOr) is.
+__device__ __forceinline__ uint32_t visited_fetch_or(uint32_t* word, uint32_t bit) {
+  return __hip_atomic_fetch_or(word, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 // marks one id visited (lane 0 does it); returns nothing, logs it for the undo
 __device__ __forceinline__ void visit_single(Scratch& s, SearchState& st, uint32_t id, int lane) {
   if (lane == 0) {
-    atomicOr(&s.bitmap[id >> 5], 1u << (id & 31));
+    visited_fetch_or(&s.bitmap[id >> 5], 1u << (id & 31));
     if (st.undo_cnt < s.undo_cap) s.undo[st.undo_cnt] = id;
   }
   st.undo_cnt += 1;
@@ -257,7 +291,7 @@ __device__ __forceinline__ int visit_row(const uint32_t* row, int S, Scratch& s,
     bool newly = false;
     if (id != kEmpty) {
       uint32_t bit = 1u << (id & 31);
-      uint32_t old = atomicOr(&s.bitmap[id >> 5], bit);
+      uint32_t old = visited_fetch_or(&s.bitmap[id >> 5], bit);
       newly = (old & bit) == 0;
     }
     unsigned long long mask = __ballot(newly);
@@ -305,16 +339,20 @@ __device__ __forceinline__ void undo_visited(Scratch& s, SearchState& st, int la
 // "push, then pop the maximum" becomes one sorted insert (about 35 vector instructions, no
 // LDS).  Which ids survive is decided at the end from the log of accepted entries; only a
 // tie exactly at the k-th key needs the literal heap, which is then replayed from the log.
-// Unused positions hold +inf; when the set is full, evicted keys drift to positions >= ef,
-// where they are never read and never counted (they are >= the bound that admitted v).
+// Unused positions hold +inf; when the set is full the evicted key falls off the end.
 template <int NS>
 struct TopKeys {
   float k[NS > 0 ? NS : 1];
 };
+// The keys are kept right-aligned: sorted position p lives in physical slot p + 64*NS - ef,
+// the slots below hold -inf and never move.  The largest key of a FULL set then always sits
+// in the last slot of lane 63 — a fixed register, which matters: indexing the register
+// array with a run-time position would push it through scratch memory.
 template <int NS>
-__device__ __forceinline__ void topkeys_init(TopKeys<NS>& t) {
+__device__ __forceinline__ void topkeys_init(TopKeys<NS>& t, int ef, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
 #pragma unroll
-  for (int j = 0; j < (NS > 0 ? NS : 1); ++j) t.k[j] = INFINITY;
+  for (int j = 0; j < N; ++j) t.k[j] = (lane * N + j < 64 * N - ef) ? -INFINITY : INFINITY;
 }
 template <int NS>
 __device__ __forceinline__ void topkeys_insert(TopKeys<NS>& t, float v, int lane) {
@@ -335,15 +373,23 @@ __device__ __forceinline__ void topkeys_insert(TopKeys<NS>& t, float v, int lane
     t.k[j] = j > pos ? below : (j == pos ? incoming : t.k[j]);
   }
 }
-// key at sorted position pos (wavefront-uniform)
+// largest key of a full set
 template <int NS>
-__device__ __forceinline__ float topkeys_at(const TopKeys<NS>& t, int pos) {
+__device__ __forceinline__ float topkeys_max(const TopKeys<NS>& t) {
   constexpr int N = NS > 0 ? NS : 1;
-  const int l = pos / N, r = pos - l * N;
-  float x = t.k[0];
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t.k[N - 1]), 63));
+}
+// key at sorted position pos (wavefront-uniform, once per search): through an LDS copy
+template <int NS>
+__device__ __forceinline__ float topkeys_at(const TopKeys<NS>& t, int pos, int ef, float* lds_tmp, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+  wave_sync();
 #pragma unroll
-  for (int j = 1; j < N; ++j) x = r == j ? t.k[j] : x;
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l));
+  for (int j = 0; j < N; ++j) lds_tmp[lane * N + j] = t.k[j];
+  wave_sync();
+  const float x = lds_tmp[pos + 64 * N - ef];
+  wave_sync();
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
 }
 
 // Offers nbuf/dbuf[0..n) in stored order (hnswlib's accept rule, identical to the
@@ -386,7 +432,8 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
       if (NS > 0) {
         topkeys_insert<NS>(tk, e.key, lane);
         st.top_size = st.n_acc < ef ? st.n_acc : ef;
-        st.lower = topkeys_at<NS>(tk, st.top_size - 1);
+        st.maxkey = fmaxf(st.maxkey, e.key);
+        st.lower = st.n_acc >= ef ? topkeys_max<NS>(tk) : st.maxkey;  // hnswlib's lowerBound
       } else {
         LdsHeap top{s.top};
         coop_push<false>(top, st.top_size, e, lane);

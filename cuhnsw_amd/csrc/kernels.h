@@ -126,10 +126,10 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     QVec<QR> qv;
     load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
     SearchState st;
-    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.undo_cnt = 0;
+    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY; st.undo_cnt = 0;
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
     TopKeys<NS> tk;
-    topkeys_init<NS>(tk);
+    topkeys_init<NS>(tk, a.ef, lane);
 
     uint32_t cur = ix.enterpoint;
     float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
@@ -147,7 +147,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     bool literal = NS == 0;
     if (NS > 0 && !st.fail) {
       __threadfence_block();
-      const float bound = topkeys_at<NS>(tk, T - 1);
+      const float bound = topkeys_at<NS>(tk, T - 1, a.ef, reinterpret_cast<float*>(s.cand), lane);
       const int cnt = collect_le(s.log, st.n_acc, bound, s.top, a.lcap, lane);
       if (cnt != T) {
         literal = true;
@@ -293,10 +293,10 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     QVec<QR> qv;
     load_node_query<QR>(qv, s.qlds, ix, x, lane);
     SearchState st;
-    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.undo_cnt = 0;
+    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY; st.undo_cnt = 0;
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
     TopKeys<NS> tk;
-    topkeys_init<NS>(tk);
+    topkeys_init<NS>(tk, a.efc, lane);
     visit_single(s, st, x, lane);  // a node never links to itself
 
     int n_seed = 0;
@@ -327,7 +327,8 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     int T = st.top_size;
     if (NS > 0 && T > 0) {
       __threadfence_block();
-      T = collect_best(s.log, st.n_acc, topkeys_at<NS>(tk, T - 1), T, s.top, lane);
+      const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
+      T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
     }
     wave_sync();
     rank_sort(s.top, nullptr, T, sid, skey, lane);
