@@ -191,9 +191,15 @@ __device__ __forceinline__ void dist_pass(const float4* rows, int rowlen, const 
   for (int u = 0; u < U; ++u) {
     const int idx = r + 4 * u + g;
     const uint32_t id = ids[idx < n ? idx : n - 1];
-    const float4* p = rows + (size_t)id * rowlen + sub;
+    const float4* p = rows + (size_t)id * rowlen;
 #pragma unroll
-    for (int k = 0; k < R; ++k) v[u][k] = (sub + 16 * k < rowlen) ? p[16 * k] : zero;
+    for (int k = 0; k < R; ++k) {
+      // always one unconditional 16-byte load (a guarded one is split into four dword loads);
+      // chunks past the row end re-read chunk 0 and are zeroed afterwards
+      const int c = sub + 16 * k;
+      const float4 t = p[c < rowlen ? c : 0];
+      v[u][k] = c < rowlen ? t : zero;
+    }
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -240,12 +246,16 @@ __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv
     for (int r = 0; r < n; r += 4) {
       const int idx = r + g;
       const uint32_t id = ids[idx < n ? idx : n - 1];
-      const float4* p = rows + (size_t)id * rowlen + sub;
+      const float4* p = rows + (size_t)id * rowlen;
       float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
       for (int k0 = 0; k0 < nk; k0 += B) {
         float4 v[B];
 #pragma unroll
-        for (int b = 0; b < B; ++b) v[b] = (sub + 16 * (k0 + b) < rowlen) ? p[16 * (k0 + b)] : zero;
+        for (int b = 0; b < B; ++b) {
+          const int c = sub + 16 * (k0 + b);
+          const float4 t = p[c < rowlen ? c : 0];  // unconditional 16-byte load
+          v[b] = c < rowlen ? t : zero;
+        }
 #pragma unroll
         for (int b = 0; b < B; ++b) {
           // chunks past the row end multiply zeros (the LDS copy is padded to a multiple of 16

@@ -216,7 +216,11 @@ __device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, cons
   if (QR > 0) {
     const int sub = lane & 15;
 #pragma unroll
-    for (int k = 0; k < (QR > 0 ? QR : 1); ++k) qv.q[k] = (sub + 16 * k < rowlen) ? p[sub + 16 * k] : zero;
+    for (int k = 0; k < (QR > 0 ? QR : 1); ++k) {
+      const int c = sub + 16 * k;
+      const float4 t = p[c < rowlen ? c : 0];  // unconditional 16-byte load
+      qv.q[k] = c < rowlen ? t : zero;
+    }
   } else {
     const int chunks = (rowlen + 15) / 16 * 16;
     wave_sync();
