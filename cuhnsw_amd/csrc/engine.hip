@@ -161,12 +161,25 @@ class Engine {
     return rc;
   }
 
+  // vectors go up as one contiguous copy (a pitched copy from pageable memory crawls row by
+  // row); rows that need padding are spread out by a small kernel on the device
   void upload_vectors() {
     Dp = padded_dims(host.D);
-    d_vectors.reserve((size_t)host.N * Dp);
-    HIP_CHECK(hipMemsetAsync(d_vectors.p, 0, (size_t)host.N * Dp * sizeof(float), stream));
-    HIP_CHECK(hipMemcpy2DAsync(d_vectors.p, (size_t)Dp * 4, host.vectors.data(), (size_t)host.D * 4, (size_t)host.D * 4,
-                               (size_t)host.N, hipMemcpyHostToDevice, stream));
+    const size_t n = (size_t)host.N;
+    d_vectors.reserve(n * Dp);
+    if (Dp == host.D) {
+      HIP_CHECK(hipMemcpyAsync(d_vectors.p, host.vectors.data(), n * Dp * sizeof(float), hipMemcpyHostToDevice, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+      return;
+    }
+    DevBuf<float> raw;
+    raw.reserve(n * host.D);
+    HIP_CHECK(hipMemcpyAsync(raw.p, host.vectors.data(), n * host.D * sizeof(float), hipMemcpyHostToDevice, stream));
+    HIP_CHECK(hipMemsetAsync(d_vectors.p, 0, n * Dp * sizeof(float), stream));
+    const long long work = (long long)n * host.D;
+    hipLaunchKernelGGL(pad_rows_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, raw.p, d_vectors.p,
+                       (long long)n, host.D, Dp);
+    HIP_CHECK(hipGetLastError());
     HIP_CHECK(hipStreamSynchronize(stream));
   }
 

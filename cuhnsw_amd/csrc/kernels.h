@@ -241,14 +241,20 @@ __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32
   int head = 0;
   int tail = (m < T ? m : T) - 1;
   const int max_head = tail + 1;
+  // candidates are examined in list order whatever the outcome, so the next candidate's
+  // vector can be fetched while the current one is being tested (register copy; for long
+  // rows the LDS copy is filled when the candidate comes up)
+  QVec<QR> cv_next;
+  if (QR > 0 && T > 0) load_node_query<QR>(cv_next, s.qlds, ix, sid[0], lane);
   for (int j = 0; j < T; ++j) {
     if (head >= m) break;
     const uint32_t c = sid[j];
     const float dq = skey[j];
     bool skip = false;
+    QVec<QR> cv = cv_next;
+    if (QR > 0 && j + 1 < T) load_node_query<QR>(cv_next, s.qlds, ix, sid[j + 1], lane);
     if (head >= nn_num && head > 0) {
-      QVec<QR> cv;
-      load_node_query<QR>(cv, s.qlds, ix, c, lane);
+      if (QR == 0) load_node_query<QR>(cv, s.qlds, ix, c, lane);
       dist_list<DT, QR, false>(ix, cv, s.qlds, oid, head, s.dbuf, lane);
       wave_sync();
       bool mine = false;
@@ -479,6 +485,15 @@ __global__ void __launch_bounds__(256) inherit_kernel(DevIndex ix, int level, co
   }
   link_row_mut(ix, x, level)[j] = id;
   dist_row_mut(ix, x, level)[j] = key;
+}
+
+// Upload helper: copies N x D floats into rows of Dp floats (the padding was zeroed before).
+__global__ void __launch_bounds__(256) pad_rows_kernel(const float* src, float* dst, long long n, int D, int Dp) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * D) return;
+  const long long row = i / D;
+  const int col = (int)(i - row * D);
+  dst[row * Dp + col] = src[i];
 }
 
 }  // namespace cuhnsw_amd
