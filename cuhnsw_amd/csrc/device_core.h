@@ -53,6 +53,8 @@ struct Scratch {
   uint32_t* nbuf;      // LDS, lcap ids
   float* dbuf;         // LDS, lcap keys
   float4* qlds;        // LDS copy of the query (only when the query is not kept in registers)
+  uint16_t* vcache;    // LDS, direct-mapped cache of ids known to be visited (null = none)
+  int vc_bits;         // log2 of its size: slot = id & (size-1), tag = id >> vc_bits
   uint32_t* bitmap;    // global, one bit per node
   uint32_t* undo;      // global, ids whose bit is set
   int undo_cap;
@@ -283,11 +285,25 @@ __device__ __forceinline__ uint32_t visited_fetch_or(uint32_t* word, uint32_t bi
   return __hip_atomic_fetch_or(word, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
+// In front of the bitmap sits a small direct-mapped cache in LDS of ids already known to be
+// visited (16-bit tags, slot = low id bits).  Most neighbours of an expanded node were seen
+// a few hops earlier; a cache hit answers "visited" exactly (tags are only written for ids
+// whose bit is set) and saves the global atomic — on the 1.18M-point benchmark the atomics
+// were more than half of all L2 requests and nearly all of the DRAM write traffic.
+__device__ __forceinline__ void vcache_reset(Scratch& s, int lane) {
+  if (s.vcache == nullptr) return;
+  uint4* c4 = reinterpret_cast<uint4*>(s.vcache);
+  const int n4 = (1 << s.vc_bits) >> 3;  // 8 tags per 16 bytes
+  for (int i = lane; i < n4; i += 64) c4[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+  wave_sync();
+}
+
 // marks one id visited (lane 0 does it); returns nothing, logs it for the undo
 __device__ __forceinline__ void visit_single(Scratch& s, SearchState& st, uint32_t id, int lane) {
   if (lane == 0) {
     visited_fetch_or(&s.bitmap[id >> 5], 1u << (id & 31));
     if (st.undo_cnt < s.undo_cap) s.undo[st.undo_cnt] = id;
+    if (s.vcache != nullptr) s.vcache[id & ((1u << s.vc_bits) - 1u)] = (uint16_t)(id >> s.vc_bits);
   }
   st.undo_cnt += 1;
 }
@@ -298,11 +314,20 @@ __device__ __forceinline__ int visit_row(const uint32_t* row, int S, Scratch& s,
   int n = 0;
   for (int base = 0; base < S; base += 64) {
     uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
+    bool ask = id != kEmpty;
+    uint32_t slot = 0;
+    uint16_t tag = 0;
+    if (s.vcache != nullptr && ask) {
+      slot = id & ((1u << s.vc_bits) - 1u);
+      tag = (uint16_t)(id >> s.vc_bits);
+      ask = s.vcache[slot] != tag;  // hit: visited for sure
+    }
     bool newly = false;
-    if (id != kEmpty) {
+    if (ask) {
       uint32_t bit = 1u << (id & 31);
       uint32_t old = visited_fetch_or(&s.bitmap[id >> 5], bit);
       newly = (old & bit) == 0;
+      if (s.vcache != nullptr) s.vcache[slot] = tag;
     }
     unsigned long long mask = __ballot(newly);
     int pos = n + __popcll(mask & ((1ull << lane) - 1ull));
@@ -312,6 +337,7 @@ __device__ __forceinline__ int visit_row(const uint32_t* row, int S, Scratch& s,
       if (u < s.undo_cap) s.undo[u] = id;
     }
     n += __popcll(mask);
+    wave_sync();
   }
   st.undo_cnt += n;
   return n;

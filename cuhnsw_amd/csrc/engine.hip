@@ -79,6 +79,7 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  int visited_cache = 0;  // entries of the LDS visited cache: 0 = automatic, < 0 = none
   // 1 = when a level is built, nodes that also live above are searched and re-selected
   // again like the new ones (the reference processes every node of a level,
   // cpp/include/cuda_build_kernels.cuh:188).  Off by default: replacing their rows
@@ -283,6 +284,17 @@ class Engine {
     return std::max(c, std::max(floor_entries, 128));
   }
 
+  // log2 entries of the LDS visited cache (16-bit tags: usable while N >> bits fits 16 bits
+  // with 0xFFFF to spare)
+  int auto_vc_bits() const {
+    if (visited_cache < 0) return 0;
+    int want = visited_cache > 0 ? visited_cache : 1024;
+    int bits = 8;
+    while ((1 << bits) < want && bits < 14) ++bits;
+    if (((unsigned)host.N >> bits) >= 0xFFFFu) return 0;
+    return bits;
+  }
+
   template <typename K>
   int resident_slots(K kernel, size_t lds) const {
     int per_cu = 0;
@@ -294,7 +306,7 @@ class Engine {
   // ---- search ------------------------------------------------------------------------------
   template <int DT, int QR, int NS>
   void launch_search(const DevIndex& ix, SearchArgs& a, int max_slots_override, float* ms) {
-    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0);
+    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
     auto kernel = search_kernel<DT, QR, NS>;
     int slots = resident_slots(kernel, lp.total);
     if (max_slots_override > 0) slots = max_slots_override;
@@ -354,6 +366,7 @@ class Engine {
     const int q = qr();
     size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
     const int ns = key_slots(ef);
+    a.vc_bits = auto_vc_bits();
     // with the keys in registers the queue's LDS share doubles as result buffer (lcap entries,
     // then lcap label slots) and as the replay heap (ef + 1 entries)
     const int floor_entries = ns > 0 ? std::max(ef + 1, 2 * a.lcap) : std::max(k, 64);
@@ -462,7 +475,8 @@ class Engine {
       size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_cap * 8 + 64 +
                      (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
       a.cand_lds = auto_cand_lds(efc, NS, 64, fixed);
-      const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_cap);
+      a.vc_bits = auto_vc_bits();
+      const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_cap, a.vc_bits);
       const LdsPlan lp3 = plan_lds(QR, Dp, S + cap_in, 0, a.lcap, S + cap_in, m_cap);
       const int slots1 = resident_slots(k_search, lp1.total);
       const int slots3 = resident_slots(k_reverse, lp3.total);
@@ -648,6 +662,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "cand_lds") e->impl.cand_lds_override = (int)value;
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
   else if (n == "reprocess_upper") e->impl.reprocess_upper = (int)value;
+  else if (n == "visited_cache") e->impl.visited_cache = (int)value;
   else return -1;
   return 0;
 }

@@ -44,6 +44,7 @@ struct SearchArgs {
   int* status;   // set to 1 when a candidate queue ran out of room
   SlotPool pool;
   int cand_lds, lcap, hnswlib_dist;
+  int vc_bits;  // log2 entries of the LDS visited cache, 0 = none
 };
 
 struct BuildArgs {
@@ -58,6 +59,7 @@ struct BuildArgs {
   int* status;
   SlotPool pool;
   int cand_lds, lcap;
+  int vc_bits;
   HeapEnt* inbox;  // N x cap_in
   int* inbox_cnt;  // N
   int cap_in;
@@ -69,9 +71,10 @@ __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t
 
 // LDS layout of one wavefront (shared by host sizing and device carving)
 struct LdsPlan {
-  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, total;
+  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, vcache, total;
 };
-__host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds, int lcap, int n_sorted, int n_out) {
+__host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds, int lcap, int n_sorted, int n_out,
+                                            int vc_bits = 0) {
   LdsPlan p;
   size_t o = 0;
   p.qlds = o;
@@ -84,6 +87,7 @@ __host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds
   p.out_key = o; o = align16(o + (size_t)n_out * 4);
   p.nbuf = o; o = align16(o + (size_t)lcap * 4);
   p.dbuf = o; o = align16(o + (size_t)lcap * 4);
+  p.vcache = o; o = align16(o + (vc_bits > 0 ? ((size_t)2 << vc_bits) : 0));
   p.total = o;
   return p;
 }
@@ -104,8 +108,10 @@ template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
   Scratch s;
+  s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
+  s.vc_bits = a.vc_bits;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
   s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
@@ -130,6 +136,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
     TopKeys<NS> tk;
     topkeys_init<NS>(tk, a.ef, lane);
+    vcache_reset(s, lane);
 
     uint32_t cur = ix.enterpoint;
     float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
@@ -279,8 +286,10 @@ template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, a.efc, a.cand_lds, a.lcap, a.efc, a.m_cap);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, a.efc, a.cand_lds, a.lcap, a.efc, a.m_cap, a.vc_bits);
   Scratch s;
+  s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
+  s.vc_bits = a.vc_bits;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
   s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
@@ -307,6 +316,7 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
     TopKeys<NS> tk;
     topkeys_init<NS>(tk, a.efc, lane);
+    vcache_reset(s, lane);
     visit_single(s, st, x, lane);  // a node never links to itself
 
     int n_seed = 0;

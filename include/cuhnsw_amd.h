@@ -100,6 +100,8 @@ double cuhnsw_last_build_seconds(cuhnsw_engine* e);
  *   "search_slots"  resident wavefronts used by search (0 = automatic)
  *   "cand_lds"      candidate-queue entries kept in LDS (0 = automatic)
  *   "hnswlib_dist"  1 = return hnswlib distances (1-dot) instead of -dot
+ *   "visited_cache" entries of the LDS cache in front of the visited bitmap (0 = automatic,
+ *                   negative = none)
  *   "reprocess_upper" 1 = also re-insert, on every level, the nodes that live on
  *                   higher levels too (default 0: they keep inherited + reverse links)
  * returns non-zero for an unknown name */
