@@ -85,7 +85,8 @@ def test_search_parity_on_oracle_built_index(oracle, tmp_path, name, n, d, dist,
   e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=max_m0)
   e.load_index(p)
   assert (e.num_data, e.num_dims, e.max_level, e.enter_point) == (n, d, ix.maxlevel, ix.enterpoint)
-  for k, ef in ((10, 300), (1, 1), (10, 10), (100, 64), (100, 120), (7, 33)):
+  # ef < 320: result keys in 5 registers per lane; < 1024: 16 registers; beyond: literal LDS heap
+  for k, ef in ((10, 300), (1, 1), (10, 10), (100, 64), (100, 120), (7, 33), (10, 400), (50, 1023), (10, 1100)):
     _check_parity(oracle, ix, e, q, k, ef)
 
 
@@ -166,6 +167,9 @@ def test_candidate_queue_spills_to_global_memory(oracle, tmp_path):
   _check_parity(oracle, ix, e, q, 10, 400)
   e.set_tunable("search_slots", 3)  # many queries per resident wavefront: visited sets must be clean between queries
   _check_parity(oracle, ix, e, q, 10, 100)
+  for entries in (-1, 256, 8192):   # without / tiny / large LDS visited cache: same answers
+    e.set_tunable("visited_cache", entries)
+    _check_parity(oracle, ix, e, q, 10, 100)
 
 
 def test_errors(tmp_path):
