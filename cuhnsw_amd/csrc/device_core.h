@@ -343,6 +343,54 @@ __device__ __forceinline__ int visit_row(const uint32_t* row, int S, Scratch& s,
   return n;
 }
 
+// The same for rows of at most 64 slots, split in two so that the vector rows of the
+// neighbours can be fetched WHILE the visited atomics are in flight instead of after them:
+// visit_issue() starts the atomics for every neighbour the cache does not vouch for and
+// compacts those ids into s.nbuf; the caller computes their distances; visit_commit() then
+// reads the atomics' answers, blanks the entries that turn out to have been visited before
+// (kEmpty in s.nbuf; their distances are discarded) and logs the new ones for the undo.
+// The speculative rows are few: after the cache most remaining neighbours are new.
+struct VisitPending {
+  uint32_t id, bit, old;
+  int pos, n_ask;
+  bool ask;
+};
+__device__ __forceinline__ VisitPending visit_issue(const uint32_t* row, int S, Scratch& s, int lane) {
+  VisitPending v;
+  v.id = lane < S ? row[lane] : kEmpty;
+  v.ask = v.id != kEmpty;
+  uint32_t slot = 0;
+  uint16_t tag = 0;
+  if (s.vcache != nullptr && v.ask) {
+    slot = v.id & ((1u << s.vc_bits) - 1u);
+    tag = (uint16_t)(v.id >> s.vc_bits);
+    v.ask = s.vcache[slot] != tag;
+  }
+  const unsigned long long mask = __ballot(v.ask);
+  v.pos = __popcll(mask & ((1ull << lane) - 1ull));
+  v.n_ask = __popcll(mask);
+  v.bit = 1u << (v.id & 31);
+  v.old = 0u;
+  if (v.ask) {
+    v.old = visited_fetch_or(&s.bitmap[v.id >> 5], v.bit);
+    s.nbuf[v.pos] = v.id;
+    if (s.vcache != nullptr) s.vcache[slot] = tag;
+  }
+  return v;
+}
+__device__ __forceinline__ int visit_commit(const VisitPending& v, Scratch& s, SearchState& st, int lane) {
+  const bool newly = v.ask && (v.old & v.bit) == 0u;
+  const unsigned long long mask = __ballot(newly);
+  if (v.ask && !newly) s.nbuf[v.pos] = kEmpty;
+  if (newly) {
+    const int u = st.undo_cnt + __popcll(mask & ((1ull << lane) - 1ull));
+    if (u < s.undo_cap) s.undo[u] = v.id;
+  }
+  const int n_new = __popcll(mask);
+  st.undo_cnt += n_new;
+  return n_new;
+}
+
 // Reads a link row and compacts its valid ids into s.nbuf without touching the visited set.
 __device__ __forceinline__ int load_row(const uint32_t* row, int S, Scratch& s, int lane) {
   int n = 0;
@@ -437,13 +485,14 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
   for (int base = 0; base < n; base += 64) {
-    // every lane takes one offer; offers that already fail against the current bound can
-    // be dropped at once (the bound never rises once the set is full), the others are
-    // taken in stored order and re-checked against the bound as it moves
+    // every lane takes one offer; blanked entries (speculatively fetched neighbours that had
+    // been visited before) and offers that already fail against the current bound are
+    // dropped at once (the bound never rises once the set is full), the others are taken in
+    // stored order and re-checked against the bound as it moves
     const int mine = base + lane;
     const float my_key = mine < n ? s.dbuf[mine] : INFINITY;
     const uint32_t my_id = mine < n ? s.nbuf[mine] : 0u;
-    unsigned long long todo = __ballot(mine < n && (st.top_size < ef || st.lower > my_key));
+    unsigned long long todo = __ballot(mine < n && my_id != kEmpty && (st.top_size < ef || st.lower > my_key));
     while (todo != 0ull) {
       const int j = __builtin_ctzll(todo);
       todo &= todo - 1ull;
@@ -492,11 +541,11 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int S = row_stride(ix, level);
   int n = n_seed;
+  if (n > 0) {
+    dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    st.n_dist += n;
+  }
   while (true) {
-    if (n > 0) {
-      dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
-      st.n_dist += n;
-    }
     wave_sync();
     int cid = -1;
     accept_list<NS>(s, st, tk, n, ef, lane);
@@ -517,8 +566,20 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
     wave_sync();
     if (cid < 0) break;
     st.n_hops += 1;
-    n = visit_row(link_row(ix, (uint32_t)cid, level), S, s, st, lane);
-    wave_sync();
+    const uint32_t* row = link_row(ix, (uint32_t)cid, level);
+    if (S <= 64) {
+      const VisitPending vp = visit_issue(row, S, s, lane);
+      wave_sync();
+      n = vp.n_ask;
+      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      wave_sync();
+      st.n_dist += visit_commit(vp, s, st, lane);
+    } else {
+      n = visit_row(row, S, s, st, lane);
+      wave_sync();
+      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      st.n_dist += n;
+    }
   }
 }
 
