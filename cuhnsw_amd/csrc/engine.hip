@@ -79,6 +79,7 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  int spill_cap = 0;  // first size of the per-slot queue overflow area (0 = automatic); the accept log is twice that
   int visited_cache = 0;  // entries of the LDS visited cache: 0 = automatic, < 0 = none
   // 1 = when a level is built, nodes that also live above are searched and re-selected
   // again like the new ones (the reference processes every node of a level,
@@ -311,8 +312,8 @@ class Engine {
     int slots = resident_slots(kernel, lp.total);
     if (max_slots_override > 0) slots = max_slots_override;
     slots = std::max(1, std::min(slots, a.nq));
-    int glob_cap = std::max(4096, 8 * a.ef);
-    for (int attempt = 0; attempt < 6; ++attempt) {
+    int glob_cap = spill_cap > 0 ? spill_cap : std::max(4096, 8 * a.ef);
+    for (int attempt = 0; attempt < 8; ++attempt) {
       ensure_pool(slots, glob_cap, 2 * glob_cap);
       a.pool = pool;
       a.counter = d_ctl.p;
@@ -663,6 +664,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
   else if (n == "reprocess_upper") e->impl.reprocess_upper = (int)value;
   else if (n == "visited_cache") e->impl.visited_cache = (int)value;
+  else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else return -1;
   return 0;
 }

@@ -102,6 +102,8 @@ double cuhnsw_last_build_seconds(cuhnsw_engine* e);
  *   "hnswlib_dist"  1 = return hnswlib distances (1-dot) instead of -dot
  *   "visited_cache" entries of the LDS cache in front of the visited bitmap (0 = automatic,
  *                   negative = none)
+ *   "spill_cap"     first size (entries) of the per-wavefront queue overflow area; the search
+ *                   is repeated with four times the room when it proves too small (0 = automatic)
  *   "reprocess_upper" 1 = also re-insert, on every level, the nodes that live on
  *                   higher levels too (default 0: they keep inherited + reverse links)
  * returns non-zero for an unknown name */

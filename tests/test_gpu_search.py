@@ -172,6 +172,23 @@ def test_candidate_queue_spills_to_global_memory(oracle, tmp_path):
     _check_parity(oracle, ix, e, q, 10, 100)
 
 
+def test_overflowing_scratch_areas_are_retried(oracle, tmp_path):
+  """Accept log and queue overflow area start far too small: the engine must notice, grow
+  them and repeat the search with unchanged answers."""
+  n, d = 6000, 24
+  x = gauss_mixture(n, d, seed=13)
+  q = gauss_mixture(80, d, seed=14)
+  mult = 1 / np.log(8)
+  ix = oracle.OracleIndex("dot").build(x, _levels(n, mult, 15), 8, 16, 60, mult)
+  p = str(tmp_path / "r.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="dot", max_m=8, max_m0=16)
+  e.load_index(p)
+  e.set_tunable("spill_cap", 8)
+  _check_parity(oracle, ix, e, q, 10, 300)
+  _check_parity(oracle, ix, e, q, 10, 1200)   # literal-heap path
+
+
 def test_errors(tmp_path):
   e = _engine(tmp_path)
   e.set_data(np.zeros((8, 4), np.float32))
