@@ -80,19 +80,30 @@ def main():
   eng.build_graph()
   build_s = eng.last_build_seconds
 
-  # exact top-k on the GPU (harness only) for recall
+  # exact top-k on the GPU (harness only) for recall.  Scores are produced in blocks of at most
+  # 2^28 elements (1 GiB): larger matmul outputs came back with wrong entries on this stack.
   dd = torch.from_numpy(data).cuda()
   qq = torch.from_numpy(queries).cuda()
+  sq = (dd * dd).sum(1) if o["dist_type"] != "dot" else None
+  cols = 1 << 19
   gt = []
-  for s in range(0, nq, 500):
-    qs = qq[s:s + 500]
-    if o["dist_type"] == "dot":
-      score = -(qs @ dd.T)
-    else:
-      score = (dd * dd).sum(1)[None, :] - 2.0 * (qs @ dd.T)
-    gt.append(torch.topk(score, k, dim=1, largest=False).indices.cpu().numpy())
+  for s in range(0, nq, 512):
+    qs = qq[s:s + 512]
+    best_v = best_i = None
+    for c in range(0, n, cols):
+      score = -(qs @ dd[c:c + cols].T)
+      if sq is not None:
+        score = sq[None, c:c + cols] + 2.0 * score
+      tv, ti = torch.topk(score, min(k, score.shape[1]), dim=1, largest=False)
+      ti = ti + c
+      if best_v is not None:
+        tv, ti = torch.cat([best_v, tv], 1), torch.cat([best_i, ti], 1)
+        tv, sel = torch.topk(tv, min(k, tv.shape[1]), dim=1, largest=False)
+        ti = torch.gather(ti, 1, sel)
+      best_v, best_i = tv, ti
+    gt.append(best_i.cpu().numpy())
   gt = np.concatenate(gt)
-  del dd, score
+  del dd, score, sq
 
   nns = torch.empty((nq, k), dtype=torch.int32, device="cuda")
   dist = torch.empty((nq, k), dtype=torch.float32, device="cuda")

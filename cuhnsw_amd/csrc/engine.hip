@@ -79,13 +79,9 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  int own_links0 = 0;  // links a new node selects for itself on level 0: 0 = max_m0 (as the reference), else min(value, max_m0); hnswlib uses max_m
   int spill_cap = 0;  // first size of the per-slot queue overflow area (0 = automatic); the accept log is twice that
   int visited_cache = 0;  // entries of the LDS visited cache: 0 = automatic, < 0 = none
-  // 1 = when a level is built, nodes that also live above are searched and re-selected
-  // again like the new ones (the reference processes every node of a level,
-  // cpp/include/cuda_build_kernels.cuh:188).  Off by default: replacing their rows
-  // drops reverse links they collected and measurably lowers recall on large sets.
-  int reprocess_upper = 0;
 
   // resident index
   int Dp = 0;
@@ -399,43 +395,31 @@ class Engine {
     const int N = host.N;
     const int cap_in = 32;
     const int bmax = std::max(1, build_batch);
-    DevBuf<float> d_dists0, d_distsU, d_sel_keys;
-    DevBuf<uint32_t> d_sel_ids, d_dirty;
-    DevBuf<int> d_sel_cnt, d_inbox_cnt, d_level_nodes;
-    DevBuf<HeapEnt> d_inbox;
-    const int m_cap_max = std::max(host.max_m, host.max_m0);
+    const int m_max = std::max(host.max_m, host.max_m0);
+    const size_t up_rows = std::max<size_t>((size_t)host.upper_rows, 1);
+    DevBuf<float> d_dists0, d_distsU, d_sel0_keys, d_selU_keys;
+    DevBuf<uint32_t> d_sel0_ids, d_selU_ids;
+    DevBuf<unsigned long long> d_dirty;
+    DevBuf<int> d_sel0_cnt, d_selU_cnt, d_inbox0_cnt, d_inboxU_cnt;
+    DevBuf<HeapEnt> d_inbox0, d_inboxU;
     d_dists0.reserve((size_t)N * host.S0);
-    d_distsU.reserve(std::max<size_t>((size_t)host.upper_rows * host.SU, 1));
-    d_sel_ids.reserve((size_t)bmax * m_cap_max);
-    d_sel_keys.reserve((size_t)bmax * m_cap_max);
-    d_sel_cnt.reserve((size_t)bmax);
-    d_dirty.reserve((size_t)bmax * m_cap_max);
-    d_inbox.reserve((size_t)N * cap_in);
-    d_inbox_cnt.reserve((size_t)N);
-    HIP_CHECK(hipMemsetAsync(d_inbox_cnt.p, 0, (size_t)N * 4, stream));
+    d_distsU.reserve(up_rows * host.SU);
+    d_sel0_ids.reserve((size_t)bmax * host.max_m0);
+    d_sel0_keys.reserve((size_t)bmax * host.max_m0);
+    d_sel0_cnt.reserve((size_t)bmax);
+    d_selU_ids.reserve(up_rows * host.max_m);
+    d_selU_keys.reserve(up_rows * host.max_m);
+    d_selU_cnt.reserve(up_rows);
+    // a batch node posts at most max_m0 links on level 0 and max_m on each upper level
+    d_dirty.reserve((size_t)bmax * ((size_t)host.max_m0 + (size_t)std::max(host.maxlevel, 1) * host.max_m));
+    d_inbox0.reserve((size_t)N * cap_in);
+    d_inbox0_cnt.reserve((size_t)N);
+    d_inboxU.reserve(up_rows * cap_in);
+    d_inboxU_cnt.reserve(up_rows);
+    HIP_CHECK(hipMemsetAsync(d_inbox0_cnt.p, 0, (size_t)N * 4, stream));
+    HIP_CHECK(hipMemsetAsync(d_inboxU_cnt.p, 0, up_rows * 4, stream));
     HIP_CHECK(hipMemsetAsync(d_links0.p, 0xFF, (size_t)N * host.S0 * 4, stream));
     if (host.upper_rows > 0) HIP_CHECK(hipMemsetAsync(d_linksU.p, 0xFF, (size_t)host.upper_rows * host.SU * 4, stream));
-
-    // ascending node lists of the upper levels, concatenated
-    std::vector<std::vector<int>> lists(host.maxlevel + 1);
-    for (int i = 0; i < N; ++i)
-      for (int l = 1; l <= host.levels[i]; ++l) lists[l].push_back(i);
-    std::vector<size_t> list_off(host.maxlevel + 2, 0), new_off(host.maxlevel + 2, 0);
-    std::vector<int> new_cnt(host.maxlevel + 2, 0);
-    std::vector<int> flat;
-    for (int l = 1; l <= host.maxlevel; ++l) {
-      list_off[l] = flat.size();
-      flat.insert(flat.end(), lists[l].begin(), lists[l].end());
-    }
-    for (int l = 0; l <= host.maxlevel; ++l) {
-      new_off[l] = flat.size();
-      if (!reprocess_upper)
-        for (int i = 0; i < N; ++i)
-          if (host.levels[i] == l) flat.push_back(i);
-      new_cnt[l] = (int)(flat.size() - new_off[l]);
-    }
-    d_level_nodes.reserve(std::max<size_t>(flat.size(), 1));
-    if (!flat.empty()) HIP_CHECK(hipMemcpyAsync(d_level_nodes.p, flat.data(), flat.size() * 4, hipMemcpyHostToDevice, stream));
 
     DevIndex ix = dev_index(d_dists0.p, d_distsU.p);
     auto k_search = build_search_kernel<DT, QR, NS>;
@@ -443,65 +427,63 @@ class Engine {
     const int efc = opt.ef_construction;
     const int glob_cap = std::max(4096, 8 * efc);
 
-    for (int lv = host.maxlevel; lv >= 0; --lv) {
-      int n_lv = lv == 0 ? N : (int)lists[lv].size();
-      const int* nodes = lv == 0 ? nullptr : d_level_nodes.p + list_off[lv];
-      if (!reprocess_upper) {
-        n_lv = new_cnt[lv];
-        nodes = d_level_nodes.p + new_off[lv];
-      }
-      const int S = lv == 0 ? host.S0 : host.SU;
-      const int m_cap = lv == 0 ? host.max_m0 : host.max_m;
-      int n_skel = 0;
-      if (lv < host.maxlevel) {
-        n_skel = (int)lists[lv + 1].size();
-        long long work = (long long)n_skel * S;
-        hipLaunchKernelGGL(inherit_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, ix, lv,
-                           d_level_nodes.p + list_off[lv + 1], n_skel);
-        HIP_CHECK(hipGetLastError());
-      }
-      BuildArgs a{};
-      a.level = lv;
-      a.level_nodes = nodes;
-      a.efc = efc;
-      a.m_cap = m_cap;
-      a.nn_num = (int)(m_cap * opt.heuristic_coef);
-      a.save_remains = opt.save_remains ? 1 : 0;
-      a.sel_ids = d_sel_ids.p; a.sel_keys = d_sel_keys.p; a.sel_cnt = d_sel_cnt.p;
-      a.counter = d_ctl.p; a.status = d_ctl.p + 1;
-      a.inbox = d_inbox.p; a.inbox_cnt = d_inbox_cnt.p; a.cap_in = cap_in;
-      a.dirty = d_dirty.p; a.dirty_cnt = d_ctl.p + 2;
-      a.lcap = (std::max(S, 64) + 63) / 64 * 64;
-      const int q = QR;
-      size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_cap * 8 + 64 +
-                     (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
-      a.cand_lds = auto_cand_lds(efc, NS, 64, fixed);
-      a.vc_bits = auto_vc_bits();
-      const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_cap, a.vc_bits);
-      const LdsPlan lp3 = plan_lds(QR, Dp, S + cap_in, 0, a.lcap, S + cap_in, m_cap);
-      const int slots1 = resident_slots(k_search, lp1.total);
-      const int slots3 = resident_slots(k_reverse, lp3.total);
-      ensure_pool(slots1, glob_cap, 2 * glob_cap);
-      a.pool = pool;
+    BuildArgs a{};
+    a.efc = efc;
+    a.nn_num0 = (int)(host.max_m0 * opt.heuristic_coef);
+    a.nn_numU = (int)(host.max_m * opt.heuristic_coef);
+    a.save_remains = opt.save_remains ? 1 : 0;
+    a.own_cap0 = own_links0 > 0 ? std::min(own_links0, host.max_m0) : host.max_m0;
+    a.sel0_ids = d_sel0_ids.p; a.sel0_keys = d_sel0_keys.p; a.sel0_cnt = d_sel0_cnt.p;
+    a.selU_ids = d_selU_ids.p; a.selU_keys = d_selU_keys.p; a.selU_cnt = d_selU_cnt.p;
+    a.counter = d_ctl.p; a.status = d_ctl.p + 1;
+    a.inbox0 = d_inbox0.p; a.inbox0_cnt = d_inbox0_cnt.p;
+    a.inboxU = d_inboxU.p; a.inboxU_cnt = d_inboxU_cnt.p;
+    a.cap_in = cap_in;
+    a.dirty = d_dirty.p; a.dirty_cnt = d_ctl.p + 2;
+    const int s_max = std::max(host.S0, host.SU);
+    a.lcap = (std::max(s_max, 64) + 63) / 64 * 64;
+    size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_max * 8 + 64 +
+                   (QR == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
+    a.cand_lds = auto_cand_lds(efc, NS, 64, fixed);
+    a.vc_bits = auto_vc_bits();
+    const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_max, a.vc_bits);
+    const LdsPlan lp3 = plan_lds(QR, Dp, s_max + cap_in, 0, a.lcap, s_max + cap_in, m_max);
+    const int slots1 = resident_slots(k_search, lp1.total);
+    const int slots3 = resident_slots(k_reverse, lp3.total);
+    ensure_pool(slots1, glob_cap, 2 * glob_cap);
+    a.pool = pool;
 
-      int pos = 0;
-      while (pos < n_lv) {
-        int b = std::max(1, std::min(bmax, (n_skel + pos) / 4));
-        b = std::min(b, n_lv - pos);
-        a.begin = pos;
-        a.count = b;
-        // counter and dirty count back to zero; the status word is sticky
-        HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, sizeof(int), stream));
-        HIP_CHECK(hipMemsetAsync(d_ctl.p + 2, 0, sizeof(int), stream));
-        hipLaunchKernelGGL(k_search, dim3(std::min(b, slots1)), dim3(64), lp1.total, stream, ix, a);
-        HIP_CHECK(hipGetLastError());
-        long long work = (long long)b * m_cap;
+    // Nodes go in by ascending id, as hnswlib inserts them.  The graph a batch sees is the
+    // one of all earlier batches: its entry point is the first node that reached the highest
+    // level so far.  Batches grow with the graph (a quarter of what is already in) up to
+    // build_batch, so that early nodes, which wire the long-range links, see each other.
+    int cur_ep = 0, cur_max = -1;
+    int pos = 0;
+    while (pos < N) {
+      int b = std::max(1, std::min(bmax, pos / 4));
+      b = std::min(b, N - pos);
+      a.begin = pos;
+      a.count = b;
+      a.cur_ep = cur_ep;
+      a.cur_max = cur_max;
+      // counter and dirty count back to zero; the status word is sticky
+      HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, sizeof(int), stream));
+      HIP_CHECK(hipMemsetAsync(d_ctl.p + 2, 0, sizeof(int), stream));
+      hipLaunchKernelGGL(k_search, dim3(std::min(b, slots1)), dim3(64), lp1.total, stream, ix, a);
+      HIP_CHECK(hipGetLastError());
+      if (cur_max >= 0) {
+        long long work = (long long)b * m_max;
         hipLaunchKernelGGL(apply_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, ix, a);
         HIP_CHECK(hipGetLastError());
         hipLaunchKernelGGL(k_reverse, dim3((unsigned)std::min<long long>(work, slots3)), dim3(64), lp3.total, stream, ix, a);
         HIP_CHECK(hipGetLastError());
-        pos += b;
       }
+      for (int i = pos; i < pos + b; ++i)
+        if (host.levels[i] > cur_max) {
+          cur_max = host.levels[i];
+          cur_ep = i;
+        }
+      pos += b;
     }
     int ctl[4];
     HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
@@ -662,8 +644,8 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "search_slots") e->impl.search_slots = (int)value;
   else if (n == "cand_lds") e->impl.cand_lds_override = (int)value;
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
-  else if (n == "reprocess_upper") e->impl.reprocess_upper = (int)value;
   else if (n == "visited_cache") e->impl.visited_cache = (int)value;
+  else if (n == "own_links0") e->impl.own_links0 = (int)value;
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else return -1;
   return 0;

@@ -6,15 +6,20 @@
 //                      level-0 ef-search for a whole query batch.
 // build_search_kernel, apply_kernel, reverse_kernel
 //                      replace BuildLevelGraphKernel + SearchHeuristic
-//                      (cpp/include/cuda_build_kernels.cuh:68-338).  The reference
-//                      inserts all nodes of a level concurrently under per-node spin
-//                      locks; here a level is inserted in batches of three lock-free
-//                      phases separated by kernel boundaries:
-//                        1. every node of the batch searches the frozen graph and
-//                           selects its neighbours (read-only on the graph),
-//                        2. the selections are written and each chosen neighbour y
-//                           receives the newcomer in y's inbox,
-//                        3. one wavefront per touched y merges inbox and row (append
+//                      (cpp/include/cuda_build_kernels.cuh:68-338) and the per-level host
+//                      orchestration (cpp/src/cuhnsw_build.cu:96-208).  The reference builds
+//                      level by level, top down, every node of a level concurrently under
+//                      per-node spin locks.  Here nodes are inserted in id order, each on all
+//                      of its levels at once (hnswlib's order: early nodes leave long-range
+//                      links on level 0, which is what keeps strongly clustered sets
+//                      navigable), in batches of three lock-free phases separated by kernel
+//                      boundaries:
+//                        1. every node of the batch descends from the current entry point,
+//                           searches each of its levels on the frozen graph and selects its
+//                           neighbours there (read-only on the graph),
+//                        2. the selections are written and each chosen neighbour y receives
+//                           the newcomer in y's inbox of that level,
+//                        3. one wavefront per touched (y, level) merges inbox and row (append
 //                           while there is room, else the selection heuristic).
 //                      The result is deterministic for a given batch schedule.
 #pragma once
@@ -48,22 +53,27 @@ struct SearchArgs {
 };
 
 struct BuildArgs {
-  int level;
-  const int* level_nodes;  // ascending ids of the nodes of this level, null = identity
-  int begin, count;        // batch = level_nodes[begin .. begin+count)
-  int efc, m_cap, nn_num, save_remains;
-  uint32_t* sel_ids;  // count x m_cap
-  float* sel_keys;
-  int* sel_cnt;
+  int begin, count;        // batch = nodes begin .. begin+count-1
+  int cur_ep, cur_max;     // entry point and top level of the graph before this batch (cur_max < 0: empty)
+  int efc, nn_num0, nn_numU, save_remains;
+  int own_cap0;  // how many links a new node may choose for itself on level 0 (<= max_m0)
+  uint32_t* sel0_ids;  // count x max_m0: level-0 selections of the batch
+  float* sel0_keys;
+  int* sel0_cnt;
+  uint32_t* selU_ids;  // upper rows x max_m: upper-level selections, indexed like linksU rows
+  float* selU_keys;
+  int* selU_cnt;
   int* counter;
   int* status;
   SlotPool pool;
   int cand_lds, lcap;
   int vc_bits;
-  HeapEnt* inbox;  // N x cap_in
-  int* inbox_cnt;  // N
+  HeapEnt* inbox0;  // N x cap_in
+  int* inbox0_cnt;  // N
+  HeapEnt* inboxU;  // upper rows x cap_in
+  int* inboxU_cnt;  // upper rows
   int cap_in;
-  uint32_t* dirty;
+  unsigned long long* dirty;  // node | level << 32
   int* dirty_cnt;
 };
 
@@ -286,7 +296,8 @@ template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, a.efc, a.cand_lds, a.lcap, a.efc, a.m_cap, a.vc_bits);
+  const int m_max = ix.max_m0 > ix.max_m ? ix.max_m0 : ix.max_m;
+  const LdsPlan lp = plan_lds(QR, ix.Dp, a.efc, a.cand_lds, a.lcap, a.efc, m_max, a.vc_bits);
   Scratch s;
   s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
   s.vc_bits = a.vc_bits;
@@ -308,62 +319,71 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     if (lane == 0) b = atomicAdd(a.counter, 1);
     b = __builtin_amdgcn_readfirstlane(b);
     if (b >= a.count) break;
-    const uint32_t x = a.level_nodes ? (uint32_t)a.level_nodes[a.begin + b] : (uint32_t)(a.begin + b);
+    const uint32_t x = (uint32_t)(a.begin + b);
+    const int lx = ix.levels[x];
+    const int top_level = lx < a.cur_max ? lx : a.cur_max;  // levels x shares with the graph so far
+    if (lane == 0) a.sel0_cnt[b] = 0;
+    if (top_level < 0) continue;  // very first node: nothing to link to
     QVec<QR> qv;
     load_node_query<QR>(qv, s.qlds, ix, x, lane);
     SearchState st;
-    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY; st.undo_cnt = 0;
-    st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
-    TopKeys<NS> tk;
-    topkeys_init<NS>(tk, a.efc, lane);
-    vcache_reset(s, lane);
-    visit_single(s, st, x, lane);  // a node never links to itself
+    st.undo_cnt = 0; st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
 
-    int n_seed = 0;
-    if (ix.levels[x] == a.level) {
-      // first appearance of x: enter through the finished upper levels
-      if (a.level == ix.maxlevel) {
-        if (x != ix.enterpoint) {
-          visit_single(s, st, ix.enterpoint, lane);
-          if (lane == 0) s.nbuf[0] = ix.enterpoint;
-          n_seed = 1;
-        }
-      } else {
-        uint32_t cur = ix.enterpoint;
-        float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
-        descend<DT, QR>(ix, qv, ix.maxlevel, a.level, cur, dcur, s, st, lane);
-        visit_single(s, st, cur, lane);
-        if (lane == 0) s.nbuf[0] = cur;
-        n_seed = 1;
+    // hnswlib addPoint: greedy descent from the entry point down to the node's top level,
+    // then search + select on every level it has, entering each level at the closest
+    // neighbour chosen one level up
+    uint32_t cur = (uint32_t)a.cur_ep;
+    if (a.cur_max > lx) {
+      float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
+      descend<DT, QR>(ix, qv, a.cur_max, lx, cur, dcur, s, st, lane);
+    }
+    for (int level = top_level; level >= 0; --level) {
+      const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
+      st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY;
+      TopKeys<NS> tk;
+      topkeys_init<NS>(tk, a.efc, lane);
+      vcache_reset(s, lane);
+      visit_single(s, st, x, lane);  // a node never links to itself
+      visit_single(s, st, cur, lane);
+      if (lane == 0) s.nbuf[0] = cur;
+      wave_sync();
+      search_level<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, tk, 1, lane);
+
+      // the efc best accepted entries (any deterministic choice among equal keys at the cut)
+      int T = st.top_size;
+      if (NS > 0 && T > 0) {
+        __threadfence_block();
+        const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
+        T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
       }
-    } else {
-      // x also lives above: start from the links it inherited at this level
-      n_seed = visit_row(link_row(ix, x, a.level), row_stride(ix, a.level), s, st, lane);
+      wave_sync();
+      rank_sort(s.top, nullptr, T, sid, skey, lane);
+      wave_sync();
+      const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, level == 0 ? a.own_cap0 : m_cap,
+                                               level == 0 ? a.nn_num0 : a.nn_numU, a.save_remains, oid, okey, s, lane);
+      if (QR == 0) load_node_query<QR>(qv, s.qlds, ix, x, lane);  // the LDS query copy was reused by the selection
+      uint32_t* out_ids;
+      float* out_keys;
+      if (level == 0) {
+        out_ids = a.sel0_ids + (size_t)b * ix.max_m0;
+        out_keys = a.sel0_keys + (size_t)b * ix.max_m0;
+        if (lane == 0) a.sel0_cnt[b] = deg;
+      } else {
+        const size_t r = (size_t)(ix.upper_off[x] + level - 1);
+        out_ids = a.selU_ids + r * ix.max_m;
+        out_keys = a.selU_keys + r * ix.max_m;
+        if (lane == 0) a.selU_cnt[r] = deg;
+      }
+      for (int j = lane; j < m_cap; j += 64) {
+        out_ids[j] = j < deg ? oid[j] : kEmpty;
+        out_keys[j] = j < deg ? okey[j] : 0.f;
+      }
+      if (deg > 0) cur = oid[0];  // closest selected neighbour: entry for the level below
+      wave_sync();
+      undo_visited(s, st, lane);
+      wave_sync();
     }
-    wave_sync();
-    search_level<DT, QR, NS, true>(ix, qv, a.level, a.efc, s, st, tk, n_seed, lane);
-
-    // the efc best accepted entries (any deterministic choice among equal keys at the cut)
-    int T = st.top_size;
-    if (NS > 0 && T > 0) {
-      __threadfence_block();
-      const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
-      T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
-    }
-    wave_sync();
-    rank_sort(s.top, nullptr, T, sid, skey, lane);
-    wave_sync();
-    const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);
-    for (int j = lane; j < a.m_cap; j += 64) {
-      a.sel_ids[(size_t)b * a.m_cap + j] = j < deg ? oid[j] : kEmpty;
-      a.sel_keys[(size_t)b * a.m_cap + j] = j < deg ? okey[j] : 0.f;
-    }
-    if (lane == 0) {
-      a.sel_cnt[b] = deg;
-      if (st.fail) *a.status = 1;
-    }
-    undo_visited(s, st, lane);
-    wave_sync();
+    if (lane == 0 && st.fail) *a.status = 1;
   }
 }
 
@@ -374,38 +394,69 @@ __device__ __forceinline__ float* dist_row_mut(const DevIndex& ix, uint32_t node
   return level == 0 ? ix.dists0 + (size_t)node * ix.S0 : ix.distsU + (size_t)(ix.upper_off[node] + level - 1) * ix.SU;
 }
 
-// Phase 2: write the selected rows and post the reverse links.
+// Phase 2: write the selected rows and post the reverse links.  Thread (b, j) handles slot j
+// of node b on each of its levels.
 __global__ void __launch_bounds__(256) apply_kernel(DevIndex ix, BuildArgs a) {
+  const int m_max = ix.max_m0 > ix.max_m ? ix.max_m0 : ix.max_m;
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= (long long)a.count * a.m_cap) return;
-  const int b = (int)(i / a.m_cap), j = (int)(i % a.m_cap);
-  const uint32_t x = a.level_nodes ? (uint32_t)a.level_nodes[a.begin + b] : (uint32_t)(a.begin + b);
-  const int deg = a.sel_cnt[b];
-  const uint32_t y = j < deg ? a.sel_ids[i] : kEmpty;
-  const float key = a.sel_keys[i];
-  link_row_mut(ix, x, a.level)[j] = y;
-  dist_row_mut(ix, x, a.level)[j] = key;
-  if (j < deg) {
-    int slot = atomicAdd(&a.inbox_cnt[y], 1);
-    if (slot < a.cap_in) {
-      HeapEnt e;
-      e.key = key;
-      e.id = x;
-      a.inbox[(size_t)y * a.cap_in + slot] = e;
+  if (i >= (long long)a.count * m_max) return;
+  const int b = (int)(i / m_max), j = (int)(i % m_max);
+  const uint32_t x = (uint32_t)(a.begin + b);
+  const int lx = ix.levels[x];
+  const int top_level = lx < a.cur_max ? lx : a.cur_max;
+  for (int level = 0; level <= top_level; ++level) {
+    const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
+    if (j >= m_cap) continue;
+    const uint32_t* sel_ids;
+    const float* sel_keys;
+    int deg;
+    if (level == 0) {
+      sel_ids = a.sel0_ids + (size_t)b * ix.max_m0;
+      sel_keys = a.sel0_keys + (size_t)b * ix.max_m0;
+      deg = a.sel0_cnt[b];
+    } else {
+      const size_t r = (size_t)(ix.upper_off[x] + level - 1);
+      sel_ids = a.selU_ids + r * ix.max_m;
+      sel_keys = a.selU_keys + r * ix.max_m;
+      deg = a.selU_cnt[r];
     }
-    if (slot == 0) a.dirty[atomicAdd(a.dirty_cnt, 1)] = y;
+    const uint32_t y = j < deg ? sel_ids[j] : kEmpty;
+    const float key = sel_keys[j];
+    link_row_mut(ix, x, level)[j] = y;
+    dist_row_mut(ix, x, level)[j] = key;
+    if (j < deg) {
+      int* cnt;
+      HeapEnt* box;
+      if (level == 0) {
+        cnt = a.inbox0_cnt + y;
+        box = a.inbox0 + (size_t)y * a.cap_in;
+      } else {
+        const size_t ry = (size_t)(ix.upper_off[y] + level - 1);
+        cnt = a.inboxU_cnt + ry;
+        box = a.inboxU + ry * a.cap_in;
+      }
+      const int slot = atomicAdd(cnt, 1);
+      if (slot < a.cap_in) {
+        HeapEnt e;
+        e.key = key;
+        e.id = x;
+        box[slot] = e;
+      }
+      if (slot == 0) a.dirty[atomicAdd(a.dirty_cnt, 1)] = (unsigned long long)y | ((unsigned long long)level << 32);
+    }
   }
 }
 
-// Phase 3: one wavefront per node that received reverse links.
+// Phase 3: one wavefront per (node, level) that received reverse links.
 template <int DT, int QR>
 __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const int S = row_stride(ix, a.level);
-  const int ncand = S + a.cap_in;
+  const int s_max = ix.S0 > ix.SU ? ix.S0 : ix.SU;
+  const int m_max = ix.max_m0 > ix.max_m ? ix.max_m0 : ix.max_m;
+  const int ncand = s_max + a.cap_in;
   // plan: "top" region holds the merged candidates, sorted_* their ranking
-  const LdsPlan lp = plan_lds(QR, ix.Dp, ncand, 0, a.lcap, ncand, a.m_cap);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, ncand, 0, a.lcap, ncand, m_max);
   Scratch s;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   HeapEnt* cbuf = reinterpret_cast<HeapEnt*>(smem + lp.top);
@@ -418,11 +469,25 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
   const int n_dirty = *a.dirty_cnt;
 
   for (int di = blockIdx.x; di < n_dirty; di += gridDim.x) {
-    const uint32_t y = a.dirty[di];
-    int nin = a.inbox_cnt[y];
+    const unsigned long long entry = a.dirty[di];
+    const uint32_t y = (uint32_t)(entry & 0xffffffffull);
+    const int level = (int)(entry >> 32);
+    const int S = row_stride(ix, level);
+    const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
+    int* cnt;
+    const HeapEnt* box;
+    if (level == 0) {
+      cnt = a.inbox0_cnt + y;
+      box = a.inbox0 + (size_t)y * a.cap_in;
+    } else {
+      const size_t ry = (size_t)(ix.upper_off[y] + level - 1);
+      cnt = a.inboxU_cnt + ry;
+      box = a.inboxU + ry * a.cap_in;
+    }
+    int nin = *cnt;
     nin = nin < a.cap_in ? nin : a.cap_in;
-    uint32_t* row = link_row_mut(ix, y, a.level);
-    float* drow = dist_row_mut(ix, y, a.level);
+    uint32_t* row = link_row_mut(ix, y, level);
+    float* drow = dist_row_mut(ix, y, level);
     // existing links
     int n0 = 0;
     for (int base = 0; base < S; base += 64) {
@@ -442,7 +507,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       e.key = 0.f; e.id = kEmpty;
       bool keep = false;
       if (base + lane < nin) {
-        e = a.inbox[(size_t)y * a.cap_in + base + lane];
+        e = box[base + lane];
         keep = true;
         for (int t = 0; t < n0; ++t) keep = keep && (cbuf[t].id != e.id);
       }
@@ -454,7 +519,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
     wave_sync();
     const int n_new = T - n0;
     if (n_new > 0) {
-      if (T <= a.m_cap) {
+      if (T <= m_cap) {
         // room for all: append the newcomers, ordered by (key, id)
         rank_sort(cbuf + n0, nullptr, n_new, sid, skey, lane);
         wave_sync();
@@ -465,36 +530,17 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       } else {
         rank_sort(cbuf, nullptr, T, sid, skey, lane);
         wave_sync();
-        const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, a.m_cap, a.nn_num, a.save_remains, oid, okey, s, lane);
-        for (int j = lane; j < a.m_cap; j += 64) {
+        const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, m_cap, level == 0 ? a.nn_num0 : a.nn_numU,
+                                                 a.save_remains, oid, okey, s, lane);
+        for (int j = lane; j < m_cap; j += 64) {
           row[j] = j < deg ? oid[j] : kEmpty;
           drow[j] = j < deg ? okey[j] : 0.f;
         }
       }
     }
-    if (lane == 0) a.inbox_cnt[y] = 0;
+    if (lane == 0) *cnt = 0;
     wave_sync();
   }
-}
-
-// Start of a level: every node that also lives on level+1 inherits its links from there
-// (the reference does the same on the host, cpp/src/cuhnsw_build.cu:113-125; here the
-// link keys travel with the ids).
-__global__ void __launch_bounds__(256) inherit_kernel(DevIndex ix, int level, const int* upper_nodes, int count) {
-  const int S = level == 0 ? ix.S0 : ix.SU;
-  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= (long long)count * S) return;
-  const uint32_t x = (uint32_t)upper_nodes[i / S];
-  const int j = (int)(i % S);
-  const size_t src = (size_t)(ix.upper_off[x] + level) * ix.SU;  // row of level + 1
-  uint32_t id = kEmpty;
-  float key = 0.f;
-  if (j < ix.SU) {
-    id = ix.linksU[src + j];
-    key = ix.distsU[src + j];
-  }
-  link_row_mut(ix, x, level)[j] = id;
-  dist_row_mut(ix, x, level)[j] = key;
 }
 
 // Upload helper: copies N x D floats into rows of Dp floats (the padding was zeroed before).

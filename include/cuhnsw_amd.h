@@ -104,8 +104,9 @@ double cuhnsw_last_build_seconds(cuhnsw_engine* e);
  *                   negative = none)
  *   "spill_cap"     first size (entries) of the per-wavefront queue overflow area; the search
  *                   is repeated with four times the room when it proves too small (0 = automatic)
- *   "reprocess_upper" 1 = also re-insert, on every level, the nodes that live on
- *                   higher levels too (default 0: they keep inherited + reverse links)
+ *   "own_links0"    most links a newly inserted node selects for itself on level 0
+ *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
+ *                   max_m there and max_m0 only as the room for reverse links)
  * returns non-zero for an unknown name */
 int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value);
 
