@@ -15,7 +15,7 @@ SYMBOLS = [
     "cuhnsw_save_index", "cuhnsw_load_index", "cuhnsw_search_knn",
     "cuhnsw_search_knn_device", "cuhnsw_num_data", "cuhnsw_num_dims",
     "cuhnsw_max_level", "cuhnsw_enter_point", "cuhnsw_has_device",
-    "cuhnsw_last_build_seconds", "cuhnsw_set_tunable",
+    "cuhnsw_last_build_seconds", "cuhnsw_last_search_repeats", "cuhnsw_set_tunable",
 ]
 
 _lib = None
@@ -48,6 +48,7 @@ def load():
   l.cuhnsw_has_device.argtypes = []
   l.cuhnsw_last_build_seconds.argtypes = [vp]
   l.cuhnsw_last_build_seconds.restype = cd
+  l.cuhnsw_last_search_repeats.argtypes = [vp]
   l.cuhnsw_set_tunable.argtypes = [vp, ctypes.c_char_p, cd]
   _lib = l
   return l
@@ -135,3 +136,4 @@ class Engine:
   max_level = property(lambda s: s._l.cuhnsw_max_level(s._h))
   enter_point = property(lambda s: s._l.cuhnsw_enter_point(s._h))
   last_build_seconds = property(lambda s: s._l.cuhnsw_last_build_seconds(s._h))
+  last_search_repeats = property(lambda s: s._l.cuhnsw_last_search_repeats(s._h))

@@ -583,6 +583,179 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
   }
 }
 
+// ---- the tie-free fast path -------------------------------------------------------------
+// hnswlib expands a candidate only while its key is <= lowerBound, the largest key of the
+// result set, and once an entry has been evicted from the result set its key stays >= every
+// later lowerBound.  So the candidates that are ever expanded are exactly the not yet
+// expanded members of the result set, and ONE sorted set of (key, id, expanded) does the work
+// of both priority queues (the reference's kernel uses the same view of the algorithm,
+// cpp/include/cuda_search_kernels.cuh:99-164).  The equivalence is exact as long as no two
+// keys that are in the set at the same time are equal: then the order of expansion, the
+// evicted entry and the final order do not depend on how a heap lays equal keys out.  The set
+// lives in registers, sorted, lane L holding positions [L*NS, L*NS + NS) (right-aligned like
+// TopKeys); an insert is a shift through one DPP exchange, the next candidate is the first
+// entry without the expanded mark.  An insert that meets an equal key reports it; the search
+// kernel then repeats the query with the literal queues, the build (where any deterministic
+// choice among equal keys is as good) carries on.
+template <int NS>
+struct Frontier {
+  float k[NS > 0 ? NS : 1];
+  uint32_t v[NS > 0 ? NS : 1];  // id; bit 31 = expanded (also set on the padding)
+};
+constexpr uint32_t kExpanded = 0x80000000u;
+template <int NS>
+__device__ __forceinline__ void frontier_init(Frontier<NS>& f, int ef, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    f.k[j] = (lane * N + j < 64 * N - ef) ? -INFINITY : INFINITY;
+    f.v[j] = kEmpty;
+  }
+}
+// Inserts (v, id) unless the id is already in the set (a neighbour met again after the lossy
+// visited filter forgot it).  Returns 0 = inserted, 1 = inserted next to an equal key of
+// another id, 2 = already present, nothing done.  Wavefront-uniform.
+// With a[-1] the last key of the lane below, the new key at sorted position j is the median
+// of (a[j-1], v, a[j]): a[j] where v is not below it, a[j-1] where v is below that too, else
+// v itself; the ids follow the same two comparisons.  Equal keys keep their order of arrival.
+template <int NS>
+__device__ __forceinline__ int frontier_insert(Frontier<NS>& f, float v, uint32_t id, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+  bool eq = false;
+#pragma unroll
+  for (int j = 0; j < N; ++j) eq = eq || f.k[j] == v;
+  const unsigned long long eq_mask = __ballot(eq);
+  if (eq_mask != 0ull) {
+    bool same = false;
+#pragma unroll
+    for (int j = 0; j < N; ++j) same = same || (f.k[j] == v && (f.v[j] & ~kExpanded) == id);
+    if (__ballot(same) != 0ull) return 2;
+  }
+  // last entry of the lane below (lane 0: "-inf", never taken over)
+  const float prev_k = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, f.k[N - 1]), 0x138, 0xF, 0xF, false));
+  const uint32_t prev_v = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f.v[N - 1], 0x138, 0xF, 0xF, false);
+  bool below[N + 1];  // below[j + 1]: v sorts before a[j]; below[0]: before the lane below's last
+  below[0] = v < prev_k;
+#pragma unroll
+  for (int j = 0; j < N; ++j) below[j + 1] = v < f.k[j];
+#pragma unroll
+  for (int j = N - 1; j >= 0; --j) {
+    const float lo_k = j > 0 ? f.k[j - 1] : prev_k;
+    const uint32_t lo_v = j > 0 ? f.v[j - 1] : prev_v;
+    f.k[j] = __builtin_amdgcn_fmed3f(lo_k, v, f.k[j]);
+    f.v[j] = below[j + 1] ? (below[j] ? lo_v : id) : f.v[j];
+  }
+  return eq_mask != 0ull ? 1 : 0;
+}
+template <int NS>
+__device__ __forceinline__ float frontier_max(const Frontier<NS>& f) {
+  constexpr int N = NS > 0 ? NS : 1;
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f.k[N - 1]), 63));
+}
+// closest entry not yet expanded: marks it and returns its id, or -1 when none is left
+template <int NS>
+__device__ __forceinline__ int frontier_take(Frontier<NS>& f, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+  uint32_t vf = kEmpty;
+#pragma unroll
+  for (int j = N - 1; j >= 0; --j) vf = (f.v[j] & kExpanded) == 0u ? f.v[j] : vf;
+  const unsigned long long mask = __ballot((vf & kExpanded) == 0u);
+  if (mask == 0ull) return -1;
+  const int L = __builtin_ctzll(mask);
+  const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)vf, L);
+#pragma unroll
+  for (int j = 0; j < N; ++j) f.v[j] = (lane == L && f.v[j] == id) ? (id | kExpanded) : f.v[j];
+  return (int)id;
+}
+// writes the sorted entries [0, count) to out_id / out_key (LDS)
+template <int NS>
+__device__ __forceinline__ void frontier_dump(const Frontier<NS>& f, int ef, int count, uint32_t* out_id, float* out_key,
+                                              int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const int pos = lane * N + j - (64 * N - ef);
+    if (pos >= 0 && pos < count) {
+      out_id[pos] = f.v[j] & ~kExpanded;
+      out_key[pos] = f.k[j];
+    }
+  }
+}
+
+// The fast path's visited filter: the direct-mapped tag cache in LDS alone, no bitmap.  A hit
+// is exact ("seen before"), a miss may be a node whose tag was overwritten since: it is then
+// evaluated again, which changes nothing — if it is still in the set the insert finds it, and
+// if it was rejected or evicted its key is still not below the bound.  No atomics, no global
+// memory, nothing to undo.  Compacts the ids to evaluate into s.nbuf; returns how many.
+__device__ __forceinline__ int visit_lossy(const uint32_t* row, int S, Scratch& s, int lane) {
+  int n = 0;
+  const uint32_t mask_bits = (1u << s.vc_bits) - 1u;
+  for (int base = 0; base < S; base += 64) {
+    const uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
+    bool ask = id != kEmpty;
+    if (ask) {
+      const uint32_t slot = id & mask_bits;
+      const uint16_t tag = (uint16_t)(id >> s.vc_bits);
+      ask = s.vcache[slot] != tag;
+      if (ask) s.vcache[slot] = tag;
+    }
+    const unsigned long long mask = __ballot(ask);
+    if (ask) s.nbuf[n + __popcll(mask & ((1ull << lane) - 1ull))] = id;
+    n += __popcll(mask);
+  }
+  return n;
+}
+__device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int lane) {
+  if (lane == 0) s.vcache[id & ((1u << s.vc_bits) - 1u)] = (uint16_t)(id >> s.vc_bits);
+}
+
+// Best-first search of one level on the sorted set (needs the LDS tag cache).  On entry
+// s.nbuf[0..n_seed) holds the seeds, already entered into the filter.  Returns true as soon
+// as two equal keys meet in the set (BUILD: never; the search goes on).  Nearly all such
+// pairs are two waiting candidates, whose order of expansion is the heap's choice, so giving
+// up at once wastes the least work.  On a false return fr holds the result: st.top_size
+// entries, ascending, all keys distinct.  st.n_dist counts the evaluations performed,
+// repeated ones included.
+template <int DT, int QR, int NS, bool BUILD>
+__device__ __forceinline__ bool search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
+                                                  SearchState& st, Frontier<NS>& fr, int n_seed, int lane) {
+  const int S = row_stride(ix, level);
+  int n = n_seed;
+  while (true) {
+    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    st.n_dist += n;
+    wave_sync();
+    for (int base = 0; base < n; base += 64) {
+      const int mine = base + lane;
+      const float my_key = mine < n ? s.dbuf[mine] : INFINITY;
+      const uint32_t my_id = mine < n ? s.nbuf[mine] : 0u;
+      unsigned long long todo = __ballot(mine < n && (st.n_acc < ef || st.lower > my_key));
+      while (todo != 0ull) {
+        const int j = __builtin_ctzll(todo);
+        todo &= todo - 1ull;
+        const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+        const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+        if (!(st.n_acc < ef || st.lower > key)) continue;
+        const int r = frontier_insert<NS>(fr, key, id, lane);
+        if (r == 2) continue;
+        if (!BUILD && r == 1) return true;
+        st.n_acc += 1;
+        st.maxkey = fmaxf(st.maxkey, key);
+        st.lower = st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey;  // hnswlib's lowerBound
+      }
+    }
+    st.top_size = st.n_acc < ef ? st.n_acc : ef;
+    const int cid = frontier_take<NS>(fr, lane);
+    if (cid < 0) break;
+    st.n_hops += 1;
+    wave_sync();
+    n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
+    wave_sync();
+  }
+  return false;
+}
+
 // Greedy descent through levels from_level .. to_level+1 (hnswlib searchKnn upper
 // loop; cpp/include/cuda_search_kernels.cuh:22-66 in the reference): each sweep
 // scans the neighbour list captured at its start and moves to the strictly

@@ -79,6 +79,10 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
+  bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
+  int fast_path = 1;     // 0: search with the literal queues only
+  int last_repeats = 0;  // queries of the last search that were repeated with the literal queues
   int own_links0 = 0;  // links a new node selects for itself on level 0: 0 = max_m0 (as the reference), else min(value, max_m0); hnswlib uses max_m
   int spill_cap = 0;  // first size of the per-slot queue overflow area (0 = automatic); the accept log is twice that
   int visited_cache = 0;  // entries of the LDS visited cache: 0 = automatic, < 0 = none
@@ -292,6 +296,17 @@ class Engine {
     return bits;
   }
 
+  // log2 entries of the LDS visited filter of the sorted-set search: about ten slots per
+  // result entry keep repeated evaluations rare; 0 when ids do not fit the 16-bit tags
+  int auto_fc_bits(int ef) const {
+    int want = filter_entries > 0 ? filter_entries : 10 * ef;
+    int bits = 10;
+    while ((1 << bits) < want && bits < 13) ++bits;
+    if (filter_entries > 0) { bits = 8; while ((1 << bits) < want && bits < 14) ++bits; }
+    if (((unsigned)host.N >> bits) >= 0xFFFFu) return 0;
+    return bits;
+  }
+
   template <typename K>
   int resident_slots(K kernel, size_t lds) const {
     int per_cu = 0;
@@ -303,7 +318,7 @@ class Engine {
   // ---- search ------------------------------------------------------------------------------
   template <int DT, int QR, int NS>
   void launch_search(const DevIndex& ix, SearchArgs& a, int max_slots_override, float* ms) {
-    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
+    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits, a.fc_bits);
     auto kernel = search_kernel<DT, QR, NS>;
     int slots = resident_slots(kernel, lp.total);
     if (max_slots_override > 0) slots = max_slots_override;
@@ -314,15 +329,20 @@ class Engine {
       a.pool = pool;
       a.counter = d_ctl.p;
       a.status = d_ctl.p + 1;
+      a.repeats = d_ctl.p + 3;
       HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 4 * sizeof(int), stream));
       HIP_CHECK(hipEventRecord(ev0, stream));
       hipLaunchKernelGGL(kernel, dim3(slots), dim3(64), lp.total, stream, ix, a);
       HIP_CHECK(hipGetLastError());
       HIP_CHECK(hipEventRecord(ev1, stream));
-      int ctl[2];
+      int ctl[4];
       HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
       HIP_CHECK(hipStreamSynchronize(stream));
       if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
+      last_repeats = ctl[3];
+      // an index whose distances tie all the time (integer-valued data) sends most queries
+      // through both searches: stop trying the sorted-set search on it
+      if (a.nq >= 256 && (long long)ctl[3] * 3 > a.nq) fast_suspended = true;
       if (ctl[1] == 0) return;
       scrub_pool();
       glob_cap *= 4;  // a candidate queue or accept log overflowed its global area: retry with more room
@@ -364,6 +384,8 @@ class Engine {
     size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
     const int ns = key_slots(ef);
     a.vc_bits = auto_vc_bits();
+    a.fast_path = fast_path && !fast_suspended;
+    a.fc_bits = (ns > 0 && a.fast_path) ? auto_fc_bits(ef) : 0;
     // with the keys in registers the queue's LDS share doubles as result buffer (lcap entries,
     // then lcap label slots) and as the replay heap (ef + 1 entries)
     const int floor_entries = ns > 0 ? std::max(ef + 1, 2 * a.lcap) : std::max(k, 64);
@@ -444,9 +466,11 @@ class Engine {
     a.lcap = (std::max(s_max, 64) + 63) / 64 * 64;
     size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_max * 8 + 64 +
                    (QR == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
-    a.cand_lds = auto_cand_lds(efc, NS, 64, fixed);
-    a.vc_bits = auto_vc_bits();
-    const LdsPlan lp1 = plan_lds(QR, Dp, efc, a.cand_lds, a.lcap, efc, m_max, a.vc_bits);
+    a.fc_bits = NS > 0 ? auto_fc_bits(efc) : 0;
+    const bool sorted_set = NS > 0 && a.fc_bits > 0;  // then neither queue nor literal cache is needed
+    a.cand_lds = sorted_set ? 0 : auto_cand_lds(efc, NS, 64, fixed);
+    a.vc_bits = sorted_set ? 0 : auto_vc_bits();
+    const LdsPlan lp1 = plan_lds(QR, Dp, sorted_set ? -1 : efc, a.cand_lds, a.lcap, efc, m_max, a.vc_bits, a.fc_bits);
     const LdsPlan lp3 = plan_lds(QR, Dp, s_max + cap_in, 0, a.lcap, s_max + cap_in, m_max);
     const int slots1 = resident_slots(k_search, lp1.total);
     const int slots3 = resident_slots(k_reverse, lp3.total);
@@ -524,6 +548,7 @@ class Engine {
     else build_qr<DIST_L2>(q, ns);
     last_build_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     have_graph = true;
+    fast_suspended = false;
     host_links_stale = true;
   }
 
@@ -539,6 +564,7 @@ class Engine {
     if (fresh.N <= 0) throw std::runtime_error("load_index: empty index");
     host = std::move(fresh);
     have_data = have_levels = have_graph = true;
+    fast_suspended = false;
     host_links_stale = false;
     if (has_device) {
       upload_vectors();
@@ -637,6 +663,7 @@ int cuhnsw_max_level(cuhnsw_engine* e) { return e ? e->impl.host.maxlevel : 0; }
 int cuhnsw_enter_point(cuhnsw_engine* e) { return e ? (int)e->impl.host.enterpoint : 0; }
 int cuhnsw_has_device(void) { return cuhnsw_amd::device_present() ? 1 : 0; }
 double cuhnsw_last_build_seconds(cuhnsw_engine* e) { return e ? e->impl.last_build_seconds : 0.0; }
+int cuhnsw_last_search_repeats(cuhnsw_engine* e) { return e ? e->impl.last_repeats : 0; }
 int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   if (!e || !name) return -1;
   std::string n(name);
@@ -646,6 +673,8 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
   else if (n == "visited_cache") e->impl.visited_cache = (int)value;
   else if (n == "own_links0") e->impl.own_links0 = (int)value;
+  else if (n == "fast_path") e->impl.fast_path = value != 0.0;
+  else if (n == "filter_entries") e->impl.filter_entries = (int)value;
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else return -1;
   return 0;

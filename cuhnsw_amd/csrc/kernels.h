@@ -47,9 +47,12 @@ struct SearchArgs {
   int* stats;    // nq x 4 or null
   int* counter;  // work queue head
   int* status;   // set to 1 when a candidate queue ran out of room
+  int* repeats;  // counts the queries that met equal keys and were repeated with the literal queues
   SlotPool pool;
   int cand_lds, lcap, hnswlib_dist;
-  int vc_bits;  // log2 entries of the LDS visited cache, 0 = none
+  int vc_bits;  // log2 entries of the LDS visited cache of the literal search, 0 = none
+  int fc_bits;  // log2 entries of the LDS visited filter of the sorted-set search, 0 = that search is off
+  int fast_path;  // 0 = literal queues only (exact evaluation counters)
 };
 
 struct BuildArgs {
@@ -67,7 +70,7 @@ struct BuildArgs {
   int* status;
   SlotPool pool;
   int cand_lds, lcap;
-  int vc_bits;
+  int vc_bits, fc_bits;
   HeapEnt* inbox0;  // N x cap_in
   int* inbox0_cnt;  // N
   HeapEnt* inboxU;  // upper rows x cap_in
@@ -79,25 +82,30 @@ struct BuildArgs {
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 
-// LDS layout of one wavefront (shared by host sizing and device carving)
+// LDS layout of one wavefront (shared by host sizing and device carving).  The visited
+// filter of the sorted-set search (fcache) lies over the candidate queue and the visited
+// cache of the literal search: a query uses one or the other, never both at once.
 struct LdsPlan {
-  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, vcache, total;
+  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, vcache, fcache, total;
 };
 __host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds, int lcap, int n_sorted, int n_out,
-                                            int vc_bits = 0) {
+                                            int vc_bits = 0, int fc_bits = 0) {
   LdsPlan p;
   size_t o = 0;
   p.qlds = o;
   if (qr == 0) o += (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16;
   p.top = o; o = align16(o + (size_t)(ef + 1) * 8);
   p.cand = o; o = align16(o + (size_t)cand_lds * 8);
+  p.vcache = o; o = align16(o + (vc_bits > 0 ? ((size_t)2 << vc_bits) : 0));
+  p.fcache = p.cand;
+  const size_t fend = p.fcache + (fc_bits > 0 ? ((size_t)2 << fc_bits) : 0);
+  if (fend > o) o = align16(fend);
   p.sorted_id = o; o = align16(o + (size_t)n_sorted * 4);
   p.sorted_key = o; o = align16(o + (size_t)n_sorted * 4);
   p.out_id = o; o = align16(o + (size_t)n_out * 4);
   p.out_key = o; o = align16(o + (size_t)n_out * 4);
   p.nbuf = o; o = align16(o + (size_t)lcap * 4);
   p.dbuf = o; o = align16(o + (size_t)lcap * 4);
-  p.vcache = o; o = align16(o + (vc_bits > 0 ? ((size_t)2 << vc_bits) : 0));
   p.total = o;
   return p;
 }
@@ -118,10 +126,10 @@ template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits, a.fc_bits);
   Scratch s;
-  s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
-  s.vc_bits = a.vc_bits;
+  uint16_t* const lit_cache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
+  uint16_t* const fast_cache = reinterpret_cast<uint16_t*>(smem + lp.fcache);
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
   s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
@@ -146,54 +154,84 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
     TopKeys<NS> tk;
     topkeys_init<NS>(tk, a.ef, lane);
-    vcache_reset(s, lane);
 
     uint32_t cur = ix.enterpoint;
     float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
     descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
 
-    visit_single(s, st, cur, lane);
-    if (lane == 0) s.nbuf[0] = cur;
-    wave_sync();
-    search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
-
-    // the k best.  With the keys in registers: the entries of the log at or below the k-th
-    // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the
-    // literal heap decides: replay every accepted entry through it, pop down to k.
-    int T = st.top_size < a.k ? st.top_size : a.k;
-    bool literal = NS == 0;
-    if (NS > 0 && !st.fail) {
-      __threadfence_block();
-      const float bound = topkeys_at<NS>(tk, T - 1, a.ef, reinterpret_cast<float*>(s.cand), lane);
-      const int cnt = collect_le(s.log, st.n_acc, bound, s.top, a.lcap, lane);
-      if (cnt != T) {
-        literal = true;
-        LdsHeap top{s.top};
-        int size = 0;
-        for (int i = 0; i < st.n_acc; ++i) {
-          const HeapEnt e = uniform_ent(s.log[i]);
-          coop_push<false>(top, size, e, lane);
-          if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
-        }
-        st.top_size = size;
+    bool repeated = false;
+    // First on the sorted set in registers, which is exact unless equal keys meet; in that
+    // case (and for ef beyond the register capacity) the literal queues repeat the search.
+    int T = 0;
+    bool literal_search = NS == 0 || a.fc_bits == 0 || !a.fast_path;
+    if (!literal_search) {
+      Frontier<NS> fr;
+      frontier_init<NS>(fr, a.ef, lane);
+      s.vcache = fast_cache;
+      s.vc_bits = a.fc_bits;
+      vcache_reset(s, lane);
+      visit_lossy_single(s, cur, lane);
+      if (lane == 0) s.nbuf[0] = cur;
+      wave_sync();
+      literal_search = search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane);
+      if (!literal_search) {
+        T = st.top_size < a.k ? st.top_size : a.k;
+        wave_sync();
+        frontier_dump<NS>(fr, a.ef, T, s.nbuf, s.dbuf, lane);
+        wave_sync();
+      } else {
+        repeated = true;
+        wave_sync();
+        st.top_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY; st.n_dist = 0; st.n_hops = 0;
       }
     }
-    if (literal) {
-      LdsHeap top{s.top};
-      while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
-      T = st.top_size;
-    }
-    wave_sync();
-    uint64_t* tie = nullptr;
-    if (ix.labels) {
-      // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
-      // whose first lcap entries hold the survivors themselves
-      tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
-      for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
+    if (literal_search) {
+      s.vcache = lit_cache;
+      s.vc_bits = a.vc_bits;
+      vcache_reset(s, lane);
+      visit_single(s, st, cur, lane);
+      if (lane == 0) s.nbuf[0] = cur;
+      wave_sync();
+      search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
+
+      // the k best.  With the keys in registers: the entries of the log at or below the k-th
+      // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the
+      // literal heap decides: replay every accepted entry through it, pop down to k.
+      T = st.top_size < a.k ? st.top_size : a.k;
+      bool literal = NS == 0;
+      if (NS > 0 && !st.fail) {
+        __threadfence_block();
+        const float bound = topkeys_at<NS>(tk, T - 1, a.ef, reinterpret_cast<float*>(s.cand), lane);
+        const int cnt = collect_le(s.log, st.n_acc, bound, s.top, a.lcap, lane);
+        if (cnt != T) {
+          literal = true;
+          LdsHeap top{s.top};
+          int size = 0;
+          for (int i = 0; i < st.n_acc; ++i) {
+            const HeapEnt e = uniform_ent(s.log[i]);
+            coop_push<false>(top, size, e, lane);
+            if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
+          }
+          st.top_size = size;
+        }
+      }
+      if (literal) {
+        LdsHeap top{s.top};
+        while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
+        T = st.top_size;
+      }
+      wave_sync();
+      uint64_t* tie = nullptr;
+      if (ix.labels) {
+        // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
+        // whose first lcap entries hold the survivors themselves
+        tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
+        for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
+        wave_sync();
+      }
+      rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
       wave_sync();
     }
-    rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
-    wave_sync();
     if (!a.hnswlib_dist && T > 0) {
       dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
       wave_sync();
@@ -218,6 +256,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
         a.stats[(size_t)qi * 4 + 2] = st.n_dist_upper;
         a.stats[(size_t)qi * 4 + 3] = st.n_sweeps;
       }
+      if (repeated) atomicAdd(a.repeats, 1);
     }
     undo_visited(s, st, lane);
     wave_sync();
@@ -297,10 +336,12 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
   const int m_max = ix.max_m0 > ix.max_m ? ix.max_m0 : ix.max_m;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, a.efc, a.cand_lds, a.lcap, a.efc, m_max, a.vc_bits);
+  const bool sorted_set = NS > 0 && a.fc_bits > 0;
+  const LdsPlan lp = plan_lds(QR, ix.Dp, sorted_set ? -1 : a.efc, a.cand_lds, a.lcap, a.efc, m_max, a.vc_bits, a.fc_bits);
   Scratch s;
-  s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
-  s.vc_bits = a.vc_bits;
+  s.vcache = sorted_set ? reinterpret_cast<uint16_t*>(smem + lp.fcache)
+                        : (a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr);
+  s.vc_bits = sorted_set ? a.fc_bits : a.vc_bits;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
   s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
@@ -340,25 +381,40 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     for (int level = top_level; level >= 0; --level) {
       const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
       st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY;
-      TopKeys<NS> tk;
-      topkeys_init<NS>(tk, a.efc, lane);
       vcache_reset(s, lane);
-      visit_single(s, st, x, lane);  // a node never links to itself
-      visit_single(s, st, cur, lane);
-      if (lane == 0) s.nbuf[0] = cur;
-      wave_sync();
-      search_level<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, tk, 1, lane);
-
-      // the efc best accepted entries (any deterministic choice among equal keys at the cut)
-      int T = st.top_size;
-      if (NS > 0 && T > 0) {
-        __threadfence_block();
-        const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
-        T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
+      int T;
+      if (sorted_set) {
+        // sorted set in registers: the efc best come out in order (equal keys in the order
+        // the set placed them, which is deterministic).  The new node itself cannot turn up:
+        // nothing links to it before the batch's later phases.
+        visit_lossy_single(s, cur, lane);
+        if (lane == 0) s.nbuf[0] = cur;
+        wave_sync();
+        Frontier<NS> fr;
+        frontier_init<NS>(fr, a.efc, lane);
+        search_level_fast<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, fr, 1, lane);
+        T = st.top_size;
+        wave_sync();
+        frontier_dump<NS>(fr, a.efc, T, sid, skey, lane);
+        wave_sync();
+      } else {
+        visit_single(s, st, x, lane);  // a node never links to itself
+        visit_single(s, st, cur, lane);
+        if (lane == 0) s.nbuf[0] = cur;
+        wave_sync();
+        TopKeys<NS> tk;
+        topkeys_init<NS>(tk, a.efc, lane);
+        search_level<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, tk, 1, lane);
+        T = st.top_size;
+        if (NS > 0 && T > 0) {
+          __threadfence_block();
+          const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
+          T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
+        }
+        wave_sync();
+        rank_sort(s.top, nullptr, T, sid, skey, lane);
+        wave_sync();
       }
-      wave_sync();
-      rank_sort(s.top, nullptr, T, sid, skey, lane);
-      wave_sync();
       const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, level == 0 ? a.own_cap0 : m_cap,
                                                level == 0 ? a.nn_num0 : a.nn_numU, a.save_remains, oid, okey, s, lane);
       if (QR == 0) load_node_query<QR>(qv, s.qlds, ix, x, lane);  // the LDS query copy was reused by the selection

@@ -95,6 +95,11 @@ int cuhnsw_enter_point(cuhnsw_engine* e);
 int cuhnsw_has_device(void);
 /* seconds spent inside the last cuhnsw_build_graph (device work, event-timed) */
 double cuhnsw_last_build_seconds(cuhnsw_engine* e);
+/* number of queries of the last search in which two equal distances met and which were therefore
+ * searched a second time with literal hnswlib priority queues (the first pass orders candidates
+ * by distance alone, which is exact only without ties; the reference has no such distinction
+ * because its kernel does not reproduce hnswlib's tie order) */
+int cuhnsw_last_search_repeats(cuhnsw_engine* e);
 /* tuning knobs that are not part of the reference's option table:
  *   "build_batch"   largest number of nodes inserted per batch (default 16384)
  *   "search_slots"  resident wavefronts used by search (0 = automatic)

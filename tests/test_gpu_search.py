@@ -37,19 +37,34 @@ def _device_search(e, q, k, ef):
   return nns.cpu().numpy(), dist.cpu().numpy(), found.cpu().numpy(), stats.cpu().numpy()
 
 
-def _check_parity(oracle, ix, e, q, k, ef, counters=True):
+def _check_parity(oracle, ix, e, q, k, ef, counters=True, dup_bound=3.0):
+  """Both search paths against the oracle: the default one (sorted set in registers with an
+  LDS-only visited filter; queries that meet equal keys are repeated with literal queues)
+  and the literal queues alone (fast_path = 0)."""
   o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
-  g_ids, g_d, g_f = e.search_knn(q, k, ef)
-  assert (g_f == o_f).all()
-  for r in range(q.shape[0]):
-    f = o_f[r]
-    assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d" % r
-    np.testing.assert_allclose(g_d[r, :f], o_d[r, :f], rtol=1e-5, atol=0)
-    assert (g_d[r, :f] == o_d[r, :f]).all()
-  if counters:
-    d_ids, d_d, d_f, stats = _device_search(e, q, k, ef)
-    assert (d_ids == g_ids).all() and (d_f == g_f).all()
-    assert (stats == o_cnt[:, :4]).all()
+  for fast in (1, 0):
+    e.set_tunable("fast_path", fast)
+    g_ids, g_d, g_f = e.search_knn(q, k, ef)
+    assert (g_f == o_f).all()
+    for r in range(q.shape[0]):
+      f = o_f[r]
+      assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d fast_path %d" % (r, fast)
+      np.testing.assert_allclose(g_d[r, :f], o_d[r, :f], rtol=1e-5, atol=0)
+      assert (g_d[r, :f] == o_d[r, :f]).all()
+    if counters:
+      d_ids, d_d, d_f, stats = _device_search(e, q, k, ef)
+      assert (d_ids == g_ids).all() and (d_f == g_f).all()
+      # expansions and upper-level work are the oracle's in both paths; the lossy filter of
+      # the default path may evaluate a forgotten neighbour again, the literal path never
+      assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
+      if fast:
+        assert (stats[:, 0] >= o_cnt[:, 0]).all()
+        if dup_bound:
+          assert stats[:, 0].sum() <= dup_bound * o_cnt[:, 0].sum() + 64
+      else:
+        assert (stats[:, 0] == o_cnt[:, 0]).all()
+        assert e.last_search_repeats == 0
+  e.set_tunable("fast_path", 1)
 
 
 CASES = [
@@ -170,6 +185,9 @@ def test_candidate_queue_spills_to_global_memory(oracle, tmp_path):
   for entries in (-1, 256, 8192):   # without / tiny / large LDS visited cache: same answers
     e.set_tunable("visited_cache", entries)
     _check_parity(oracle, ix, e, q, 10, 100)
+  for entries in (256, 16384):      # tiny / large visited filter of the sorted-set search
+    e.set_tunable("filter_entries", entries)
+    _check_parity(oracle, ix, e, q, 10, 100, dup_bound=None)
 
 
 def test_overflowing_scratch_areas_are_retried(oracle, tmp_path):
