@@ -683,22 +683,33 @@ __device__ __forceinline__ void frontier_dump(const Frontier<NS>& f, int ef, int
   }
 }
 
-// The fast path's visited filter: the direct-mapped tag cache in LDS alone, no bitmap.  A hit
-// is exact ("seen before"), a miss may be a node whose tag was overwritten since: it is then
-// evaluated again, which changes nothing — if it is still in the set the insert finds it, and
-// if it was rejected or evicted its key is still not below the bound.  No atomics, no global
-// memory, nothing to undo.  Compacts the ids to evaluate into s.nbuf; returns how many.
+// The sorted-set search's visited filter: a two-way set-associative tag cache in LDS alone, no
+// bitmap.  A set is one 32-bit word holding two 16-bit tags (set = low id bits, tag = the
+// rest; 0xFFFF = empty); a new tag pushes the older of the two out.  A hit is exact ("seen
+// before"), a miss may be a node whose tag has been pushed out since: it is then evaluated
+// again, which changes nothing — if it is still in the set the insert finds it, and if it was
+// rejected or evicted its key is still not below the bound.  No atomics, no global memory,
+// nothing to undo.  s.vcache / s.vc_bits hold the table and log2 of its number of sets.
+__device__ __forceinline__ void filter_reset(Scratch& s, int lane) {
+  uint4* c4 = reinterpret_cast<uint4*>(s.vcache);
+  const int n4 = (1 << s.vc_bits) >> 2;  // 4 sets per 16 bytes
+  for (int i = lane; i < n4; i += 64) c4[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+  wave_sync();
+}
+// Compacts the ids of a link row that the filter does not know into s.nbuf; returns how many.
 __device__ __forceinline__ int visit_lossy(const uint32_t* row, int S, Scratch& s, int lane) {
   int n = 0;
+  uint32_t* sets = reinterpret_cast<uint32_t*>(s.vcache);
   const uint32_t mask_bits = (1u << s.vc_bits) - 1u;
   for (int base = 0; base < S; base += 64) {
     const uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
     bool ask = id != kEmpty;
     if (ask) {
       const uint32_t slot = id & mask_bits;
-      const uint16_t tag = (uint16_t)(id >> s.vc_bits);
-      ask = s.vcache[slot] != tag;
-      if (ask) s.vcache[slot] = tag;
+      const uint32_t tag = id >> s.vc_bits;
+      const uint32_t w = sets[slot];
+      ask = (w & 0xFFFFu) != tag && (w >> 16) != tag;
+      if (ask) sets[slot] = (w << 16) | tag;
     }
     const unsigned long long mask = __ballot(ask);
     if (ask) s.nbuf[n + __popcll(mask & ((1ull << lane) - 1ull))] = id;
@@ -707,7 +718,11 @@ __device__ __forceinline__ int visit_lossy(const uint32_t* row, int S, Scratch& 
   return n;
 }
 __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int lane) {
-  if (lane == 0) s.vcache[id & ((1u << s.vc_bits) - 1u)] = (uint16_t)(id >> s.vc_bits);
+  if (lane == 0) {
+    uint32_t* sets = reinterpret_cast<uint32_t*>(s.vcache);
+    const uint32_t slot = id & ((1u << s.vc_bits) - 1u);
+    sets[slot] = (sets[slot] << 16) | (id >> s.vc_bits);
+  }
 }
 
 // Best-first search of one level on the sorted set (needs the LDS tag cache).  On entry

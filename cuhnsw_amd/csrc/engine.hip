@@ -99,7 +99,8 @@ class Engine {
   DevBuf<HeapEnt> d_cand_glob, d_log;
   SlotPool pool{};
   int pool_slots = 0;
-  DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count
+  DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count, [3] queries left for the literal pass
+  DevBuf<int> d_redo;  // their indices
   // staging for the host-pointer search entry point
   DevBuf<float> d_q, d_dist;
   DevBuf<int> d_nns, d_found;
@@ -296,13 +297,13 @@ class Engine {
     return bits;
   }
 
-  // log2 entries of the LDS visited filter of the sorted-set search: about ten slots per
-  // result entry keep repeated evaluations rare; 0 when ids do not fit the 16-bit tags
+  // log2 sets (two 16-bit tags each) of the LDS visited filter of the sorted-set search: about
+  // six entries per result entry keep repeated evaluations rare at 4 KB for ef = 300;
+  // 0 when ids do not fit the tags
   int auto_fc_bits(int ef) const {
-    int want = filter_entries > 0 ? filter_entries : 10 * ef;
-    int bits = 10;
-    while ((1 << bits) < want && bits < 13) ++bits;
-    if (filter_entries > 0) { bits = 8; while ((1 << bits) < want && bits < 14) ++bits; }
+    const int want_sets = (filter_entries > 0 ? filter_entries : 6 * ef) / 2;
+    int bits = 8;
+    while ((1 << bits) < want_sets && bits < 13) ++bits;
     if (((unsigned)host.N >> bits) >= 0xFFFFu) return 0;
     return bits;
   }
@@ -316,38 +317,67 @@ class Engine {
   }
 
   // ---- search ------------------------------------------------------------------------------
+  // Two passes: every query on the sorted set in registers (search_fast_kernel), then the
+  // queries in which equal keys met, and every query when ef exceeds the set's capacity, with
+  // the literal priority queues (search_kernel).  ms covers both.
   template <int DT, int QR, int NS>
   void launch_search(const DevIndex& ix, SearchArgs& a, int max_slots_override, float* ms) {
-    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits, a.fc_bits);
-    auto kernel = search_kernel<DT, QR, NS>;
-    int slots = resident_slots(kernel, lp.total);
-    if (max_slots_override > 0) slots = max_slots_override;
-    slots = std::max(1, std::min(slots, a.nq));
-    int glob_cap = spill_cap > 0 ? spill_cap : std::max(4096, 8 * a.ef);
-    for (int attempt = 0; attempt < 8; ++attempt) {
-      ensure_pool(slots, glob_cap, 2 * glob_cap);
-      a.pool = pool;
-      a.counter = d_ctl.p;
-      a.status = d_ctl.p + 1;
-      a.repeats = d_ctl.p + 3;
+    a.counter = d_ctl.p;
+    a.status = d_ctl.p + 1;
+    a.repeats = d_ctl.p + 3;
+    a.redo = nullptr;
+    last_repeats = 0;
+    HIP_CHECK(hipEventRecord(ev0, stream));
+    int n_literal = a.nq;
+    if (NS > 0 && a.fast_path && a.fc_bits > 0) {
+      d_redo.reserve((size_t)a.nq);
+      a.redo = d_redo.p;
+      const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
+      auto fast_kernel = search_fast_kernel<DT, QR, NS>;
+      int slots = resident_slots(fast_kernel, fp.total);
+      if (max_slots_override > 0) slots = max_slots_override;
+      slots = std::max(1, std::min(slots, a.nq));
       HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 4 * sizeof(int), stream));
-      HIP_CHECK(hipEventRecord(ev0, stream));
-      hipLaunchKernelGGL(kernel, dim3(slots), dim3(64), lp.total, stream, ix, a);
+      hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fp.total, stream, ix, a);
       HIP_CHECK(hipGetLastError());
-      HIP_CHECK(hipEventRecord(ev1, stream));
       int ctl[4];
       HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
       HIP_CHECK(hipStreamSynchronize(stream));
-      if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
-      last_repeats = ctl[3];
+      n_literal = last_repeats = ctl[3];
       // an index whose distances tie all the time (integer-valued data) sends most queries
-      // through both searches: stop trying the sorted-set search on it
-      if (a.nq >= 256 && (long long)ctl[3] * 3 > a.nq) fast_suspended = true;
-      if (ctl[1] == 0) return;
-      scrub_pool();
-      glob_cap *= 4;  // a candidate queue or accept log overflowed its global area: retry with more room
+      // through both passes: stop trying the sorted set on it
+      if (a.nq >= 256 && (long long)n_literal * 3 > a.nq) fast_suspended = true;
     }
-    throw std::runtime_error("search: candidate queue overflow");
+    if (n_literal > 0 && !getenv("CUHNSW_DEBUG_SKIP_LITERAL")) {
+      SearchArgs b = a;
+      b.nq = n_literal;
+      const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : b.ef, b.cand_lds, b.lcap, 0, 0, b.vc_bits);
+      auto kernel = search_kernel<DT, QR, NS>;
+      int slots = resident_slots(kernel, lp.total);
+      if (max_slots_override > 0) slots = max_slots_override;
+      slots = std::max(1, std::min(slots, b.nq));
+      int glob_cap = spill_cap > 0 ? spill_cap : std::max(4096, 8 * b.ef);
+      bool done = false;
+      for (int attempt = 0; attempt < 8 && !done; ++attempt) {
+        ensure_pool(slots, glob_cap, 2 * glob_cap);
+        b.pool = pool;
+        HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 3 * sizeof(int), stream));
+        hipLaunchKernelGGL(kernel, dim3(slots), dim3(64), lp.total, stream, ix, b);
+        HIP_CHECK(hipGetLastError());
+        int ctl[2];
+        HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
+        HIP_CHECK(hipStreamSynchronize(stream));
+        done = ctl[1] == 0;
+        if (!done) {
+          scrub_pool();
+          glob_cap *= 4;  // a candidate queue or accept log overflowed its global area: retry with more room
+        }
+      }
+      if (!done) throw std::runtime_error("search: candidate queue overflow");
+    }
+    HIP_CHECK(hipEventRecord(ev1, stream));
+    HIP_CHECK(hipEventSynchronize(ev1));
+    if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
   }
   template <int DT, int QR>
   void launch_search_ns(int ns, const DevIndex& ix, SearchArgs& a, float* ms) {

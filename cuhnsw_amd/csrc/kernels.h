@@ -47,11 +47,12 @@ struct SearchArgs {
   int* stats;    // nq x 4 or null
   int* counter;  // work queue head
   int* status;   // set to 1 when a candidate queue ran out of room
-  int* repeats;  // counts the queries that met equal keys and were repeated with the literal queues
+  int* repeats;  // counts the queries that met equal keys in the sorted-set pass
+  int* redo;     // their indices, for the literal pass; as input of the literal pass: the queries to answer (null = all)
   SlotPool pool;
   int cand_lds, lcap, hnswlib_dist;
   int vc_bits;  // log2 entries of the LDS visited cache of the literal search, 0 = none
-  int fc_bits;  // log2 entries of the LDS visited filter of the sorted-set search, 0 = that search is off
+  int fc_bits;  // log2 sets (two tags each) of the LDS visited filter of the sorted-set search, 0 = that search is off
   int fast_path;  // 0 = literal queues only (exact evaluation counters)
 };
 
@@ -82,9 +83,9 @@ struct BuildArgs {
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 
-// LDS layout of one wavefront (shared by host sizing and device carving).  The visited
-// filter of the sorted-set search (fcache) lies over the candidate queue and the visited
-// cache of the literal search: a query uses one or the other, never both at once.
+// LDS layout of one wavefront (shared by host sizing and device carving).  In the build's
+// search kernel the visited filter of the sorted-set search (fcache) takes the place of the
+// candidate queue and the literal search's visited cache.
 struct LdsPlan {
   size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, vcache, fcache, total;
 };
@@ -98,7 +99,7 @@ __host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds
   p.cand = o; o = align16(o + (size_t)cand_lds * 8);
   p.vcache = o; o = align16(o + (vc_bits > 0 ? ((size_t)2 << vc_bits) : 0));
   p.fcache = p.cand;
-  const size_t fend = p.fcache + (fc_bits > 0 ? ((size_t)2 << fc_bits) : 0);
+  const size_t fend = p.fcache + (fc_bits > 0 ? ((size_t)4 << fc_bits) : 0);
   if (fend > o) o = align16(fend);
   p.sorted_id = o; o = align16(o + (size_t)n_sorted * 4);
   p.sorted_key = o; o = align16(o + (size_t)n_sorted * 4);
@@ -121,15 +122,110 @@ __device__ __forceinline__ void bind_slot(Scratch& s, const SlotPool& pool, int 
   s.log_cap = pool.log_cap;
 }
 
+// LDS of the sorted-set search: query copy (long rows only), visited filter, row buffers
+struct FastLdsPlan {
+  size_t qlds, fcache, nbuf, dbuf, total;
+};
+__host__ __device__ inline FastLdsPlan plan_fast_lds(int qr, int Dp, int lcap, int fc_bits) {
+  FastLdsPlan p;
+  size_t o = 0;
+  p.qlds = o;
+  if (qr == 0) o += (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16;
+  p.fcache = o; o = align16(o + ((size_t)4 << fc_bits));
+  p.nbuf = o; o = align16(o + (size_t)lcap * 4);
+  p.dbuf = o; o = align16(o + (size_t)lcap * 4);
+  p.total = o;
+  return p;
+}
+
+// First pass of a search batch: every query on the sorted set in registers (ef < 64*NS).
+// A query in which two equal keys meet is not answered here: its index is appended to
+// a.redo (a.repeats counts them) and the literal search_kernel answers it afterwards.
+// (with five keys per lane and the query in at most two registers the kernel is held to 80
+// registers, six wavefronts per SIMD; the other shapes would spill)
+template <int DT, int QR, int NS>
+__global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x;
+  const FastLdsPlan lp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
+  Scratch s;
+  s.vcache = reinterpret_cast<uint16_t*>(smem + lp.fcache);
+  s.vc_bits = a.fc_bits;
+  s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
+  s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
+  s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
+
+  for (;;) {
+    int qi = 0;
+    if (lane == 0) qi = atomicAdd(a.counter, 1);
+    qi = __builtin_amdgcn_readfirstlane(qi);
+    if (qi >= a.nq) break;
+    QVec<QR> qv;
+    load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
+    SearchState st;
+    st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY; st.undo_cnt = 0;
+    st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
+
+    uint32_t cur = ix.enterpoint;
+    float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
+    descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
+
+    Frontier<NS> fr;
+    frontier_init<NS>(fr, a.ef, lane);
+    filter_reset(s, lane);
+    visit_lossy_single(s, cur, lane);
+    if (lane == 0) s.nbuf[0] = cur;
+    wave_sync();
+    // (the flag is made wavefront-uniform explicitly and both outcomes are plain branches)
+    const bool gave_up =
+        __builtin_amdgcn_readfirstlane((int)search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane)) != 0;
+    if (gave_up) {
+      if (lane == 0) a.redo[atomicAdd(a.repeats, 1)] = qi;
+    } else {
+      const int T = __builtin_amdgcn_readfirstlane(st.top_size < a.k ? st.top_size : a.k);
+      wave_sync();
+      frontier_dump<NS>(fr, a.ef, T, s.nbuf, s.dbuf, lane);
+      wave_sync();
+      if (!a.hnswlib_dist && T > 0) {
+        dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
+        wave_sync();
+      }
+      for (int r = lane; r < a.k; r += 64) {
+        int out_id = -1;
+        float out_d = INFINITY;
+        if (r < T) {
+          const uint32_t id = s.nbuf[r];
+          out_id = ix.labels ? (int)ix.labels[id] : (int)id;
+          out_d = s.dbuf[r];
+        }
+        a.nns[(size_t)qi * a.k + r] = out_id;
+        a.dists[(size_t)qi * a.k + r] = out_d;
+      }
+      if (lane == 0) {
+        a.found[qi] = T;
+        if (a.stats) {
+          a.stats[(size_t)qi * 4 + 0] = st.n_dist;
+          a.stats[(size_t)qi * 4 + 1] = st.n_hops;
+          a.stats[(size_t)qi * 4 + 2] = st.n_dist_upper;
+          a.stats[(size_t)qi * 4 + 3] = st.n_sweeps;
+        }
+      }
+    }
+    wave_sync();
+  }
+}
+
+// Search with literal hnswlib priority queues: the only pass for ef beyond the sorted set's
+// capacity, the second pass (over a.redo) otherwise.
 // NS > 0: result keys in registers (ef < 64*NS); NS == 0: literal result heap in LDS.
 template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits, a.fc_bits);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
   Scratch s;
-  uint16_t* const lit_cache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
-  uint16_t* const fast_cache = reinterpret_cast<uint16_t*>(smem + lp.fcache);
+  s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
+  s.vc_bits = a.vc_bits;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
   s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
@@ -147,6 +243,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     if (lane == 0) qi = atomicAdd(a.counter, 1);
     qi = __builtin_amdgcn_readfirstlane(qi);
     if (qi >= a.nq) break;
+    if (a.redo) qi = a.redo[qi];  // second pass: only the queries the sorted-set pass gave up
     QVec<QR> qv;
     load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
     SearchState st;
@@ -159,79 +256,49 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
     descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
 
-    bool repeated = false;
-    // First on the sorted set in registers, which is exact unless equal keys meet; in that
-    // case (and for ef beyond the register capacity) the literal queues repeat the search.
-    int T = 0;
-    bool literal_search = NS == 0 || a.fc_bits == 0 || !a.fast_path;
-    if (!literal_search) {
-      Frontier<NS> fr;
-      frontier_init<NS>(fr, a.ef, lane);
-      s.vcache = fast_cache;
-      s.vc_bits = a.fc_bits;
-      vcache_reset(s, lane);
-      visit_lossy_single(s, cur, lane);
-      if (lane == 0) s.nbuf[0] = cur;
-      wave_sync();
-      literal_search = search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane);
-      if (!literal_search) {
-        T = st.top_size < a.k ? st.top_size : a.k;
-        wave_sync();
-        frontier_dump<NS>(fr, a.ef, T, s.nbuf, s.dbuf, lane);
-        wave_sync();
-      } else {
-        repeated = true;
-        wave_sync();
-        st.top_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY; st.n_dist = 0; st.n_hops = 0;
-      }
-    }
-    if (literal_search) {
-      s.vcache = lit_cache;
-      s.vc_bits = a.vc_bits;
-      vcache_reset(s, lane);
-      visit_single(s, st, cur, lane);
-      if (lane == 0) s.nbuf[0] = cur;
-      wave_sync();
-      search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
+    vcache_reset(s, lane);
+    visit_single(s, st, cur, lane);
+    if (lane == 0) s.nbuf[0] = cur;
+    wave_sync();
+    search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
 
-      // the k best.  With the keys in registers: the entries of the log at or below the k-th
-      // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the
-      // literal heap decides: replay every accepted entry through it, pop down to k.
-      T = st.top_size < a.k ? st.top_size : a.k;
-      bool literal = NS == 0;
-      if (NS > 0 && !st.fail) {
-        __threadfence_block();
-        const float bound = topkeys_at<NS>(tk, T - 1, a.ef, reinterpret_cast<float*>(s.cand), lane);
-        const int cnt = collect_le(s.log, st.n_acc, bound, s.top, a.lcap, lane);
-        if (cnt != T) {
-          literal = true;
-          LdsHeap top{s.top};
-          int size = 0;
-          for (int i = 0; i < st.n_acc; ++i) {
-            const HeapEnt e = uniform_ent(s.log[i]);
-            coop_push<false>(top, size, e, lane);
-            if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
-          }
-          st.top_size = size;
-        }
-      }
-      if (literal) {
+    // the k best.  With the keys in registers: the entries of the log at or below the k-th
+    // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the
+    // literal heap decides: replay every accepted entry through it, pop down to k.
+    int T = st.top_size < a.k ? st.top_size : a.k;
+    bool literal = NS == 0;
+    if (NS > 0 && !st.fail) {
+      __threadfence_block();
+      const float bound = topkeys_at<NS>(tk, T - 1, a.ef, reinterpret_cast<float*>(s.cand), lane);
+      const int cnt = collect_le(s.log, st.n_acc, bound, s.top, a.lcap, lane);
+      if (cnt != T) {
+        literal = true;
         LdsHeap top{s.top};
-        while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
-        T = st.top_size;
+        int size = 0;
+        for (int i = 0; i < st.n_acc; ++i) {
+          const HeapEnt e = uniform_ent(s.log[i]);
+          coop_push<false>(top, size, e, lane);
+          if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
+        }
+        st.top_size = size;
       }
-      wave_sync();
-      uint64_t* tie = nullptr;
-      if (ix.labels) {
-        // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
-        // whose first lcap entries hold the survivors themselves
-        tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
-        for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
-        wave_sync();
-      }
-      rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
+    }
+    if (literal) {
+      LdsHeap top{s.top};
+      while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
+      T = st.top_size;
+    }
+    wave_sync();
+    uint64_t* tie = nullptr;
+    if (ix.labels) {
+      // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
+      // whose first lcap entries hold the survivors themselves
+      tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
+      for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
       wave_sync();
     }
+    rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
+    wave_sync();
     if (!a.hnswlib_dist && T > 0) {
       dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
       wave_sync();
@@ -256,7 +323,6 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
         a.stats[(size_t)qi * 4 + 2] = st.n_dist_upper;
         a.stats[(size_t)qi * 4 + 3] = st.n_sweeps;
       }
-      if (repeated) atomicAdd(a.repeats, 1);
     }
     undo_visited(s, st, lane);
     wave_sync();
@@ -381,9 +447,9 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     for (int level = top_level; level >= 0; --level) {
       const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
       st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY;
-      vcache_reset(s, lane);
       int T;
       if (sorted_set) {
+        filter_reset(s, lane);
         // sorted set in registers: the efc best come out in order (equal keys in the order
         // the set placed them, which is deterministic).  The new node itself cannot turn up:
         // nothing links to it before the batch's later phases.
@@ -398,6 +464,7 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
         frontier_dump<NS>(fr, a.efc, T, sid, skey, lane);
         wave_sync();
       } else {
+        vcache_reset(s, lane);
         visit_single(s, st, x, lane);  // a node never links to itself
         visit_single(s, st, cur, lane);
         if (lane == 0) s.nbuf[0] = cur;
