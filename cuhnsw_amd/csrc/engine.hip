@@ -70,6 +70,8 @@ class Engine {
   bool has_device = false;
   int num_cus = 0;
   hipStream_t stream = nullptr;
+  hipStream_t stream2 = nullptr;  // the literal pass, while the sorted-set pass runs on `stream`
+  hipEvent_t ev_side0 = nullptr, ev_side1 = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   std::string err;
   double last_build_seconds = 0.0;
@@ -79,9 +81,12 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  int side_per_cu = 4;         // its wavefronts per CU
+  int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
-  int fast_path = 1;     // 0: search with the literal queues only
+  int fast_path = 1;     // 0: search with the literal queues only; 1: sorted-set pass first when the batch is
+                         // larger than one round of literal wavefronts; 2: always
   int last_repeats = 0;  // queries of the last search that were repeated with the literal queues
   int own_links0 = 0;  // links a new node selects for itself on level 0: 0 = max_m0 (as the reference), else min(value, max_m0); hnswlib uses max_m
   int spill_cap = 0;  // first size of the per-slot queue overflow area (0 = automatic); the accept log is twice that
@@ -99,7 +104,8 @@ class Engine {
   DevBuf<HeapEnt> d_cand_glob, d_log;
   SlotPool pool{};
   int pool_slots = 0;
-  DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count, [3] queries left for the literal pass
+  DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count, [32] queries given up by the
+                      // sorted-set pass, [64] queries it has finished with, [96] work counter of a concurrent literal pass
   DevBuf<int> d_redo;  // their indices
   // staging for the host-pointer search entry point
   DevBuf<float> d_q, d_dist;
@@ -114,12 +120,18 @@ class Engine {
       HIP_CHECK(hipStreamCreate(&stream));
       HIP_CHECK(hipEventCreate(&ev0));
       HIP_CHECK(hipEventCreate(&ev1));
-      d_ctl.reserve(4);
+      d_ctl.reserve(128);
+      HIP_CHECK(hipStreamCreate(&stream2));
+      HIP_CHECK(hipEventCreate(&ev_side0));
+      HIP_CHECK(hipEventCreate(&ev_side1));
     }
   }
   ~Engine() {
     if (ev0) (void)hipEventDestroy(ev0);
     if (ev1) (void)hipEventDestroy(ev1);
+    if (ev_side0) (void)hipEventDestroy(ev_side0);
+    if (ev_side1) (void)hipEventDestroy(ev_side1);
+    if (stream2) (void)hipStreamDestroy(stream2);
     if (stream) (void)hipStreamDestroy(stream);
   }
 
@@ -297,13 +309,15 @@ class Engine {
     return bits;
   }
 
-  // log2 sets (two 16-bit tags each) of the LDS visited filter of the sorted-set search: about
-  // six entries per result entry keep repeated evaluations rare at 4 KB for ef = 300;
-  // 0 when ids do not fit the tags
+  // log2 sets (two 16-bit tags each) of the LDS visited filter of the sorted-set search.  A
+  // search evaluates about ef * max_m0 / 5 nodes; the filter gets room for somewhat more than
+  // that (4 KB at ef = 300, max_m0 = 24), and twice as much when a repeated evaluation is
+  // expensive (rows of 2 KB and more).  0 when ids do not fit the tags.
   int auto_fc_bits(int ef) const {
-    const int want_sets = (filter_entries > 0 ? filter_entries : 6 * ef) / 2;
+    long long want = filter_entries > 0 ? filter_entries : (long long)ef * host.max_m0 / 4;
+    if (filter_entries <= 0 && Dp >= 512) want *= 2;
     int bits = 8;
-    while ((1 << bits) < want_sets && bits < 13) ++bits;
+    while ((2ll << bits) < want && bits < 13) ++bits;
     if (((unsigned)host.N >> bits) >= 0xFFFFu) return 0;
     return bits;
   }
@@ -317,46 +331,86 @@ class Engine {
   }
 
   // ---- search ------------------------------------------------------------------------------
-  // Two passes: every query on the sorted set in registers (search_fast_kernel), then the
-  // queries in which equal keys met, and every query when ef exceeds the set's capacity, with
-  // the literal priority queues (search_kernel).  ms covers both.
+  // Two passes: every query on the sorted set in registers (search_fast_kernel); the queries
+  // in which equal keys met, and every query when ef exceeds the set's capacity, with the
+  // literal priority queues (search_kernel).  The literal pass normally runs at the same time
+  // on a second stream, on one wavefront per SIMD, and picks the given-up queries off a list
+  // as the first pass appends them; should it report a problem (its bounded wait ran out, or a
+  // queue overflowed) the list is answered again after the first pass.  ms covers everything.
   template <int DT, int QR, int NS>
   void launch_search(const DevIndex& ix, SearchArgs& a, int max_slots_override, float* ms) {
     a.counter = d_ctl.p;
     a.status = d_ctl.p + 1;
-    a.repeats = d_ctl.p + 3;
+    a.repeats = d_ctl.p + 32;   // the counters of the two passes sit in separate 128-byte lines
+    a.done = d_ctl.p + 64;
     a.redo = nullptr;
+    a.live = 0;
+    a.nq_total = a.nq;
+    a.slot_base = 0;
+    a.spin_limit = (int)std::min<long long>(1 << 20, std::max<long long>(1 << 14, (long long)a.nq * 8));  // about 10 us each
     last_repeats = 0;
     HIP_CHECK(hipEventRecord(ev0, stream));
+    const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
+    auto kernel = search_kernel<DT, QR, NS>;
+    int lit_slots = resident_slots(kernel, lp.total);
+    if (max_slots_override > 0) lit_slots = max_slots_override;
+    int glob_cap = spill_cap > 0 ? spill_cap : std::max(4096, 8 * a.ef);
     int n_literal = a.nq;
-    if (NS > 0 && a.fast_path && a.fc_bits > 0) {
+    bool answered = false;
+    // A batch that fits the machine in one round of literal wavefronts is latency-bound: two
+    // passes would only add the second pass's latency to the first's.
+    if (NS > 0 && a.fast_path && a.fc_bits > 0 && (a.fast_path > 1 || a.nq > lit_slots)) {
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
       const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
       auto fast_kernel = search_fast_kernel<DT, QR, NS>;
       int slots = resident_slots(fast_kernel, fp.total);
+      const bool side = concurrent_literal && max_slots_override <= 0;
+      int side_slots = 0;
+      if (side) {
+        side_slots = std::min(num_cus * side_per_cu, a.nq);
+        ensure_pool(std::max(side_slots, 1), glob_cap, 2 * glob_cap);
+        slots = std::max(num_cus, slots - num_cus * side_per_cu);  // leave the literal wavefronts their room
+      }
       if (max_slots_override > 0) slots = max_slots_override;
       slots = std::max(1, std::min(slots, a.nq));
-      HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 4 * sizeof(int), stream));
+      HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 128 * sizeof(int), stream));
+      HIP_CHECK(hipMemsetAsync(d_redo.p, 0xFF, (size_t)a.nq * sizeof(int), stream));
+      if (side) {
+        SearchArgs b = a;
+        b.live = 1;
+        b.counter = d_ctl.p + 96;
+        b.pool = pool;
+        HIP_CHECK(hipEventRecord(ev_side0, stream));
+        HIP_CHECK(hipStreamWaitEvent(stream2, ev_side0, 0));
+        hipLaunchKernelGGL(kernel, dim3(side_slots), dim3(64), lp.total, stream2, ix, b);
+        HIP_CHECK(hipGetLastError());
+        HIP_CHECK(hipEventRecord(ev_side1, stream2));
+      }
       hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fp.total, stream, ix, a);
       HIP_CHECK(hipGetLastError());
-      int ctl[4];
+      if (side) {
+        HIP_CHECK(hipStreamWaitEvent(stream, ev_side1, 0));
+      }
+      int ctl[33];
       HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
       HIP_CHECK(hipStreamSynchronize(stream));
-      n_literal = last_repeats = ctl[3];
+      n_literal = last_repeats = ctl[32];
       // an index whose distances tie all the time (integer-valued data) sends most queries
       // through both passes: stop trying the sorted set on it
       if (a.nq >= 256 && (long long)n_literal * 3 > a.nq) fast_suspended = true;
+      if (side) {
+        answered = ctl[1] == 0;
+        if (!answered) {
+          scrub_pool();
+          if (ctl[1] & 1) glob_cap *= 4;
+        }
+      }
     }
-    if (n_literal > 0 && !getenv("CUHNSW_DEBUG_SKIP_LITERAL")) {
+    if (n_literal > 0 && !answered) {
       SearchArgs b = a;
       b.nq = n_literal;
-      const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : b.ef, b.cand_lds, b.lcap, 0, 0, b.vc_bits);
-      auto kernel = search_kernel<DT, QR, NS>;
-      int slots = resident_slots(kernel, lp.total);
-      if (max_slots_override > 0) slots = max_slots_override;
-      slots = std::max(1, std::min(slots, b.nq));
-      int glob_cap = spill_cap > 0 ? spill_cap : std::max(4096, 8 * b.ef);
+      int slots = std::max(1, std::min(lit_slots, b.nq));
       bool done = false;
       for (int attempt = 0; attempt < 8 && !done; ++attempt) {
         ensure_pool(slots, glob_cap, 2 * glob_cap);
@@ -414,7 +468,7 @@ class Engine {
     size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
     const int ns = key_slots(ef);
     a.vc_bits = auto_vc_bits();
-    a.fast_path = fast_path && !fast_suspended;
+    a.fast_path = fast_suspended ? 0 : fast_path;
     a.fc_bits = (ns > 0 && a.fast_path) ? auto_fc_bits(ef) : 0;
     // with the keys in registers the queue's LDS share doubles as result buffer (lcap entries,
     // then lcap label slots) and as the replay heap (ef + 1 entries)
@@ -703,8 +757,10 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
   else if (n == "visited_cache") e->impl.visited_cache = (int)value;
   else if (n == "own_links0") e->impl.own_links0 = (int)value;
-  else if (n == "fast_path") e->impl.fast_path = value != 0.0;
+  else if (n == "fast_path") e->impl.fast_path = (int)value;
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
+  else if (n == "concurrent_literal") e->impl.concurrent_literal = value != 0.0;
+  else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(1, std::min(8, (int)value));
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else return -1;
   return 0;

@@ -49,6 +49,12 @@ struct SearchArgs {
   int* status;   // set to 1 when a candidate queue ran out of room
   int* repeats;  // counts the queries that met equal keys in the sorted-set pass
   int* redo;     // their indices, for the literal pass; as input of the literal pass: the queries to answer (null = all)
+  int* done;     // queries the sorted-set pass has finished with (answered or given up)
+  int live;      // literal pass only: 1 = the sorted-set pass is running at the same time and a.redo is
+                 // still being filled (entries start at -1); a.nq_total queries will pass through it
+  int nq_total;
+  int spin_limit;  // polls of a live literal wavefront before it gives up and reports status 2
+  int slot_base;   // first slot of the pool this launch may use (two literal launches can be in flight)
   SlotPool pool;
   int cand_lds, lcap, hnswlib_dist;
   int vc_bits;  // log2 entries of the LDS visited cache of the literal search, 0 = none
@@ -180,7 +186,10 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) s
     const bool gave_up =
         __builtin_amdgcn_readfirstlane((int)search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane)) != 0;
     if (gave_up) {
-      if (lane == 0) a.redo[atomicAdd(a.repeats, 1)] = qi;
+      if (lane == 0) {
+        const int slot = atomicAdd(a.repeats, 1);
+        __hip_atomic_store(&a.redo[slot], qi, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      }
     } else {
       const int T = __builtin_amdgcn_readfirstlane(st.top_size < a.k ? st.top_size : a.k);
       wave_sync();
@@ -211,6 +220,9 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) s
         }
       }
     }
+    // results and list entry first, then the count the literal pass watches
+    __threadfence();
+    if (lane == 0) atomicAdd(a.done, 1);
     wave_sync();
   }
 }
@@ -233,17 +245,55 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
   s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
   s.tree = make_stage_tree(lane);
-  bind_slot(s, a.pool, blockIdx.x);
+  bind_slot(s, a.pool, a.slot_base + blockIdx.x);
   // after the search the candidate queue is dead: its LDS share (>= ef + 1 entries) then
   // holds the collected results, or the literal heap when a tie has to be replayed
   if (NS > 0) s.top = s.cand;
 
   for (;;) {
     int qi = 0;
-    if (lane == 0) qi = atomicAdd(a.counter, 1);
+    if (lane == 0) {
+      qi = atomicAdd(a.counter, 1);
+      if (a.live) {
+        // entry qi of the list appears once the sorted-set pass has given up that many
+        // queries; it never will if that pass has finished them all and the entry is still
+        // empty.  The wait is bounded: past spin_limit polls the wavefront leaves with
+        // status 2 and the host answers the rest after the first pass.
+        int got = -1;
+        if (qi < a.nq_total) {
+          // every waiter polls its own list entry; the shared count is looked at only now and
+          // then, and the pauses grow, so that the waiting does not crowd the memory channel
+          // of the counters the other pass is working with
+          for (int spins = 0;; ++spins) {
+            got = __hip_atomic_load(&a.redo[qi], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+            if (got >= 0) break;
+            if ((spins & 3) == 3 &&
+                __hip_atomic_load(a.done, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) >= a.nq_total) {
+              got = __hip_atomic_load(&a.redo[qi], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+              break;
+            }
+            if (spins >= a.spin_limit) {
+              atomicOr(a.status, 2);
+              break;
+            }
+            if (spins < 16) {
+              __builtin_amdgcn_s_sleep(32);
+            } else {
+              __builtin_amdgcn_s_sleep(127);
+              __builtin_amdgcn_s_sleep(127);
+              __builtin_amdgcn_s_sleep(127);
+            }
+          }
+        }
+        qi = got;
+      } else if (qi >= a.nq) {
+        qi = -1;
+      } else if (a.redo) {
+        qi = a.redo[qi];  // second pass: only the queries the sorted-set pass gave up
+      }
+    }
     qi = __builtin_amdgcn_readfirstlane(qi);
-    if (qi >= a.nq) break;
-    if (a.redo) qi = a.redo[qi];  // second pass: only the queries the sorted-set pass gave up
+    if (qi < 0) break;
     QVec<QR> qv;
     load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
     SearchState st;
@@ -316,7 +366,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     }
     if (lane == 0) {
       a.found[qi] = st.fail ? -1 : T;
-      if (st.fail) *a.status = 1;
+      if (st.fail) atomicOr(a.status, 1);
       if (a.stats) {
         a.stats[(size_t)qi * 4 + 0] = st.n_dist;
         a.stats[(size_t)qi * 4 + 1] = st.n_hops;

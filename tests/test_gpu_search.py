@@ -42,7 +42,7 @@ def _check_parity(oracle, ix, e, q, k, ef, counters=True, dup_bound=3.0):
   LDS-only visited filter; queries that meet equal keys are repeated with literal queues)
   and the literal queues alone (fast_path = 0)."""
   o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
-  for fast in (1, 0):
+  for fast in (2, 0):   # 2 = sorted-set pass whatever the batch size
     e.set_tunable("fast_path", fast)
     g_ids, g_d, g_f = e.search_knn(q, k, ef)
     assert (g_f == o_f).all()
@@ -185,6 +185,9 @@ def test_candidate_queue_spills_to_global_memory(oracle, tmp_path):
   for entries in (-1, 256, 8192):   # without / tiny / large LDS visited cache: same answers
     e.set_tunable("visited_cache", entries)
     _check_parity(oracle, ix, e, q, 10, 100)
+  e.set_tunable("concurrent_literal", 0)   # literal pass after the sorted-set pass instead of beside it
+  _check_parity(oracle, ix, e, q, 10, 100)
+  e.set_tunable("concurrent_literal", 1)
   for entries in (256, 16384):      # tiny / large visited filter of the sorted-set search
     e.set_tunable("filter_entries", entries)
     _check_parity(oracle, ix, e, q, 10, 100, dup_bound=None)
