@@ -480,83 +480,86 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
     const int lx = ix.levels[x];
     const int top_level = lx < a.cur_max ? lx : a.cur_max;  // levels x shares with the graph so far
     if (lane == 0) a.sel0_cnt[b] = 0;
-    if (top_level < 0) continue;  // very first node: nothing to link to
-    QVec<QR> qv;
-    load_node_query<QR>(qv, s.qlds, ix, x, lane);
-    SearchState st;
-    st.undo_cnt = 0; st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
+    // (the very first node has nothing to link to; a plain branch, not a `continue` after the
+    // one-lane store above, keeps the control flow simple for the compiler)
+    if (top_level >= 0) {
+      QVec<QR> qv;
+      load_node_query<QR>(qv, s.qlds, ix, x, lane);
+      SearchState st;
+      st.undo_cnt = 0; st.n_dist = 0; st.n_hops = 0; st.n_dist_upper = 0; st.n_sweeps = 0; st.fail = 0;
 
-    // hnswlib addPoint: greedy descent from the entry point down to the node's top level,
-    // then search + select on every level it has, entering each level at the closest
-    // neighbour chosen one level up
-    uint32_t cur = (uint32_t)a.cur_ep;
-    if (a.cur_max > lx) {
-      float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
-      descend<DT, QR>(ix, qv, a.cur_max, lx, cur, dcur, s, st, lane);
-    }
-    for (int level = top_level; level >= 0; --level) {
-      const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
-      st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY;
-      int T;
-      if (sorted_set) {
-        filter_reset(s, lane);
-        // sorted set in registers: the efc best come out in order (equal keys in the order
-        // the set placed them, which is deterministic).  The new node itself cannot turn up:
-        // nothing links to it before the batch's later phases.
-        visit_lossy_single(s, cur, lane);
-        if (lane == 0) s.nbuf[0] = cur;
-        wave_sync();
-        Frontier<NS> fr;
-        frontier_init<NS>(fr, a.efc, lane);
-        search_level_fast<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, fr, 1, lane);
-        T = st.top_size;
-        wave_sync();
-        frontier_dump<NS>(fr, a.efc, T, sid, skey, lane);
-        wave_sync();
-      } else {
-        vcache_reset(s, lane);
-        visit_single(s, st, x, lane);  // a node never links to itself
-        visit_single(s, st, cur, lane);
-        if (lane == 0) s.nbuf[0] = cur;
-        wave_sync();
-        TopKeys<NS> tk;
-        topkeys_init<NS>(tk, a.efc, lane);
-        search_level<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, tk, 1, lane);
-        T = st.top_size;
-        if (NS > 0 && T > 0) {
-          __threadfence_block();
-          const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
-          T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
+      // hnswlib addPoint: greedy descent from the entry point down to the node's top level,
+      // then search + select on every level it has, entering each level at the closest
+      // neighbour chosen one level up
+      uint32_t cur = (uint32_t)a.cur_ep;
+      if (a.cur_max > lx) {
+        float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
+        descend<DT, QR>(ix, qv, a.cur_max, lx, cur, dcur, s, st, lane);
+      }
+      for (int level = top_level; level >= 0; --level) {
+        const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
+        st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY;
+        int T;
+        if (sorted_set) {
+          filter_reset(s, lane);
+          // sorted set in registers: the efc best come out in order (equal keys in the order
+          // the set placed them, which is deterministic).  The new node itself cannot turn up:
+          // nothing links to it before the batch's later phases.
+          visit_lossy_single(s, cur, lane);
+          if (lane == 0) s.nbuf[0] = cur;
+          wave_sync();
+          Frontier<NS> fr;
+          frontier_init<NS>(fr, a.efc, lane);
+          search_level_fast<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, fr, 1, lane);
+          T = st.top_size;
+          wave_sync();
+          frontier_dump<NS>(fr, a.efc, T, sid, skey, lane);
+          wave_sync();
+        } else {
+          vcache_reset(s, lane);
+          visit_single(s, st, x, lane);  // a node never links to itself
+          visit_single(s, st, cur, lane);
+          if (lane == 0) s.nbuf[0] = cur;
+          wave_sync();
+          TopKeys<NS> tk;
+          topkeys_init<NS>(tk, a.efc, lane);
+          search_level<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, tk, 1, lane);
+          T = st.top_size;
+          if (NS > 0 && T > 0) {
+            __threadfence_block();
+            const float bound = topkeys_at<NS>(tk, T - 1, a.efc, reinterpret_cast<float*>(s.cand), lane);
+            T = collect_best(s.log, st.n_acc, bound, T, s.top, lane);
+          }
+          wave_sync();
+          rank_sort(s.top, nullptr, T, sid, skey, lane);
+          wave_sync();
         }
+        const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, level == 0 ? a.own_cap0 : m_cap,
+                                                 level == 0 ? a.nn_num0 : a.nn_numU, a.save_remains, oid, okey, s, lane);
+        if (QR == 0) load_node_query<QR>(qv, s.qlds, ix, x, lane);  // the LDS query copy was reused by the selection
+        uint32_t* out_ids;
+        float* out_keys;
+        if (level == 0) {
+          out_ids = a.sel0_ids + (size_t)b * ix.max_m0;
+          out_keys = a.sel0_keys + (size_t)b * ix.max_m0;
+          if (lane == 0) a.sel0_cnt[b] = deg;
+        } else {
+          const size_t r = (size_t)(ix.upper_off[x] + level - 1);
+          out_ids = a.selU_ids + r * ix.max_m;
+          out_keys = a.selU_keys + r * ix.max_m;
+          if (lane == 0) a.selU_cnt[r] = deg;
+        }
+        for (int j = lane; j < m_cap; j += 64) {
+          out_ids[j] = j < deg ? oid[j] : kEmpty;
+          out_keys[j] = j < deg ? okey[j] : 0.f;
+        }
+        if (deg > 0) cur = oid[0];  // closest selected neighbour: entry for the level below
         wave_sync();
-        rank_sort(s.top, nullptr, T, sid, skey, lane);
+        undo_visited(s, st, lane);
         wave_sync();
       }
-      const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, level == 0 ? a.own_cap0 : m_cap,
-                                               level == 0 ? a.nn_num0 : a.nn_numU, a.save_remains, oid, okey, s, lane);
-      if (QR == 0) load_node_query<QR>(qv, s.qlds, ix, x, lane);  // the LDS query copy was reused by the selection
-      uint32_t* out_ids;
-      float* out_keys;
-      if (level == 0) {
-        out_ids = a.sel0_ids + (size_t)b * ix.max_m0;
-        out_keys = a.sel0_keys + (size_t)b * ix.max_m0;
-        if (lane == 0) a.sel0_cnt[b] = deg;
-      } else {
-        const size_t r = (size_t)(ix.upper_off[x] + level - 1);
-        out_ids = a.selU_ids + r * ix.max_m;
-        out_keys = a.selU_keys + r * ix.max_m;
-        if (lane == 0) a.selU_cnt[r] = deg;
-      }
-      for (int j = lane; j < m_cap; j += 64) {
-        out_ids[j] = j < deg ? oid[j] : kEmpty;
-        out_keys[j] = j < deg ? okey[j] : 0.f;
-      }
-      if (deg > 0) cur = oid[0];  // closest selected neighbour: entry for the level below
-      wave_sync();
-      undo_visited(s, st, lane);
-      wave_sync();
+      if (lane == 0 && st.fail) *a.status = 1;
     }
-    if (lane == 0 && st.fail) *a.status = 1;
   }
 }
 

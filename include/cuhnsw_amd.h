@@ -77,8 +77,9 @@ int cuhnsw_search_knn(cuhnsw_engine* e, const float* qdata, int num_queries, int
 /* Same search with queries and outputs already in device memory (HBM); nothing
  * is copied.  Counterpart of the kernel launch inside CuHNSW::SearchGraph
  * (cpp/src/cuhnsw_build.cu:254-275).  d_stats may be null, else int32
- * [num_queries x 4]: level-0 distance evaluations, level-0 expanded candidates,
- * upper-level distance evaluations, upper-level sweeps.  The call returns after
+ * [num_queries x 4]: level-0 distance evaluations (performed ones: the first pass may evaluate a
+ * node again after its visited filter has forgotten it; exact with tunable fast_path = 0), level-0
+ * expanded candidates, upper-level distance evaluations, upper-level sweeps.  The call returns after
  * the kernel has finished; kernel_ms (may be null) receives the kernel's duration
  * measured with HIP events on the engine's stream. */
 int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
@@ -109,6 +110,14 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   negative = none)
  *   "spill_cap"     first size (entries) of the per-wavefront queue overflow area; the search
  *                   is repeated with four times the room when it proves too small (0 = automatic)
+ *   "fast_path"     0 = search with literal hnswlib priority queues only (exact evaluation
+ *                   counters in d_stats); 1 = first pass on the sorted set in registers when the
+ *                   batch exceeds one round of resident wavefronts, literal queues for the queries
+ *                   that met equal distances (default); 2 = first pass whatever the batch size
+ *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
+ *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
+ *                   (default), 0 = after it
+ *   "literal_per_cu" wavefronts per CU of that concurrent literal pass (default 4)
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)
