@@ -81,6 +81,7 @@ class Engine {
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
+  int spin_limit_override = -1;  // polls a waiting literal wavefront may spend (-1 = automatic)
   int side_per_cu = 4;         // its wavefronts per CU
   int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
@@ -347,7 +348,9 @@ class Engine {
     a.live = 0;
     a.nq_total = a.nq;
     a.slot_base = 0;
-    a.spin_limit = (int)std::min<long long>(1 << 20, std::max<long long>(1 << 14, (long long)a.nq * 8));  // about 10 us each
+    a.spin_limit = spin_limit_override >= 0
+                       ? spin_limit_override
+                       : (int)std::min<long long>(1 << 20, std::max<long long>(1 << 14, (long long)a.nq * 8));  // about 10 us each
     last_repeats = 0;
     HIP_CHECK(hipEventRecord(ev0, stream));
     const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
@@ -760,6 +763,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "fast_path") e->impl.fast_path = (int)value;
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
   else if (n == "concurrent_literal") e->impl.concurrent_literal = value != 0.0;
+  else if (n == "literal_spin_limit") e->impl.spin_limit_override = (int)value;
   else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(1, std::min(8, (int)value));
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else return -1;

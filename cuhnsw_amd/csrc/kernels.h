@@ -261,15 +261,18 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
         // status 2 and the host answers the rest after the first pass.
         int got = -1;
         if (qi < a.nq_total) {
+          // (relaxed agent-scope loads: they read the L2 and, unlike acquire loads, do not
+          // invalidate this CU's vector cache on every poll; the list entry is the only thing
+          // read from the other pass, and it is read after the count that vouches for it)
           // every waiter polls its own list entry; the shared count is looked at only now and
           // then, and the pauses grow, so that the waiting does not crowd the memory channel
           // of the counters the other pass is working with
           for (int spins = 0;; ++spins) {
-            got = __hip_atomic_load(&a.redo[qi], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+            got = __hip_atomic_load(&a.redo[qi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (got >= 0) break;
             if ((spins & 3) == 3 &&
-                __hip_atomic_load(a.done, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) >= a.nq_total) {
-              got = __hip_atomic_load(&a.redo[qi], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_load(a.done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= a.nq_total) {
+              got = __hip_atomic_load(&a.redo[qi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
               break;
             }
             if (spins >= a.spin_limit) {

@@ -118,6 +118,8 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
  *                   (default), 0 = after it
  *   "literal_per_cu" wavefronts per CU of that concurrent literal pass (default 4)
+ *   "literal_spin_limit" polls one of its wavefronts may spend waiting for the first pass before
+ *                   it leaves and the host answers the remaining queries afterwards (-1 = automatic)
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)

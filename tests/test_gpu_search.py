@@ -193,6 +193,32 @@ def test_candidate_queue_spills_to_global_memory(oracle, tmp_path):
     _check_parity(oracle, ix, e, q, 10, 100, dup_bound=None)
 
 
+def test_literal_pass_schedules_on_tie_heavy_data(oracle, tmp_path):
+  """Integer data: most queries meet equal distances in the sorted-set pass and are answered by
+  the literal pass — beside the first pass (default), after it, and after it because the
+  waiting wavefronts were told from the host to give up at once (a bound of zero polls: every
+  kernel still ends normally)."""
+  n, d = 5000, 16
+  x = integer_vectors(n, d, seed=21, hi=30)
+  q = integer_vectors(150, d, seed=22, hi=30)
+  mult = 1 / np.log(8)
+  ix = oracle.OracleIndex("l2").build(x, _levels(n, mult, 23), 8, 16, 60, mult)
+  p = str(tmp_path / "t.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
+  e.load_index(p)
+  e.set_tunable("fast_path", 2)
+  e.search_knn(q, 10, 100)
+  assert e.last_search_repeats > 50
+  for tunable, value in (("concurrent_literal", 1), ("concurrent_literal", 0), ("literal_spin_limit", 0),
+                         ("literal_per_cu", 1)):
+    e.set_tunable("concurrent_literal", 1)
+    e.set_tunable("literal_spin_limit", -1)
+    e.set_tunable(tunable, value)
+    _check_parity(oracle, ix, e, q, 10, 100)
+    _check_parity(oracle, ix, e, q, 100, 100)
+
+
 def test_overflowing_scratch_areas_are_retried(oracle, tmp_path):
   """Accept log and queue overflow area start far too small: the engine must notice, grow
   them and repeat the search with unchanged answers."""
