@@ -653,16 +653,27 @@ __device__ __forceinline__ float frontier_max(const Frontier<NS>& f) {
   constexpr int N = NS > 0 ? NS : 1;
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f.k[N - 1]), 63));
 }
-// closest entry not yet expanded: marks it and returns its id, or -1 when none is left
+// closest (far: farthest) entry not yet expanded: marks it and returns its id, or -1 when none
+// is left.  The farthest one is what the reference expands with its reverse_cand option
+// (GetCand, cpp/include/cuda_utils_kernels.cuh:104-151).
 template <int NS>
-__device__ __forceinline__ int frontier_take(Frontier<NS>& f, int lane) {
+__device__ __forceinline__ int frontier_take(Frontier<NS>& f, int lane, bool far = false) {
   constexpr int N = NS > 0 ? NS : 1;
   uint32_t vf = kEmpty;
+  int L;
+  if (!far) {
 #pragma unroll
-  for (int j = N - 1; j >= 0; --j) vf = (f.v[j] & kExpanded) == 0u ? f.v[j] : vf;
-  const unsigned long long mask = __ballot((vf & kExpanded) == 0u);
-  if (mask == 0ull) return -1;
-  const int L = __builtin_ctzll(mask);
+    for (int j = N - 1; j >= 0; --j) vf = (f.v[j] & kExpanded) == 0u ? f.v[j] : vf;
+    const unsigned long long mask = __ballot((vf & kExpanded) == 0u);
+    if (mask == 0ull) return -1;
+    L = __builtin_ctzll(mask);
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) vf = (f.v[j] & kExpanded) == 0u ? f.v[j] : vf;
+    const unsigned long long mask = __ballot((vf & kExpanded) == 0u);
+    if (mask == 0ull) return -1;
+    L = 63 - __builtin_clzll(mask);
+  }
   const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)vf, L);
 #pragma unroll
   for (int j = 0; j < N; ++j) f.v[j] = (lane == L && f.v[j] == id) ? (id | kExpanded) : f.v[j];
@@ -731,10 +742,13 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 // pairs are two waiting candidates, whose order of expansion is the heap's choice, so giving
 // up at once wastes the least work.  On a false return fr holds the result: st.top_size
 // entries, ascending, all keys distinct.  st.n_dist counts the evaluations performed,
-// repeated ones included.
+// repeated ones included.  far: expand the farthest waiting entry instead of the closest (the
+// reference's reverse_cand); that is no hnswlib search any more, equal keys simply keep their
+// order of arrival and the query is never given up.
 template <int DT, int QR, int NS, bool BUILD>
 __device__ __forceinline__ bool search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
-                                                  SearchState& st, Frontier<NS>& fr, int n_seed, int lane) {
+                                                  SearchState& st, Frontier<NS>& fr, int n_seed, int lane,
+                                                  bool far = false) {
   const int S = row_stride(ix, level);
   int n = n_seed;
   while (true) {
@@ -754,14 +768,14 @@ __device__ __forceinline__ bool search_level_fast(const DevIndex& ix, const QVec
         if (!(st.n_acc < ef || st.lower > key)) continue;
         const int r = frontier_insert<NS>(fr, key, id, lane);
         if (r == 2) continue;
-        if (!BUILD && r == 1) return true;
+        if (!BUILD && !far && r == 1) return true;
         st.n_acc += 1;
         st.maxkey = fmaxf(st.maxkey, key);
         st.lower = st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey;  // hnswlib's lowerBound
       }
     }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
-    const int cid = frontier_take<NS>(fr, lane);
+    const int cid = frontier_take<NS>(fr, lane, far);
     if (cid < 0) break;
     st.n_hops += 1;
     wave_sync();

@@ -362,7 +362,7 @@ class Engine {
     bool answered = false;
     // A batch that fits the machine in one round of literal wavefronts is latency-bound: two
     // passes would only add the second pass's latency to the first's.
-    if (NS > 0 && a.fast_path && a.fc_bits > 0 && (a.fast_path > 1 || a.nq > lit_slots)) {
+    if (NS > 0 && a.fast_path && a.fc_bits > 0 && (a.fast_path > 1 || a.nq > lit_slots)) {  // (reverse_cand: fast_path is 2)
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
       const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
@@ -472,7 +472,11 @@ class Engine {
     const int ns = key_slots(ef);
     a.vc_bits = auto_vc_bits();
     a.fast_path = fast_suspended ? 0 : fast_path;
+    a.reverse = opt.reverse_cand ? 1 : 0;
+    if (a.reverse) a.fast_path = 2;  // only the sorted set can expand its farthest entry
     a.fc_bits = (ns > 0 && a.fast_path) ? auto_fc_bits(ef) : 0;
+    if (a.reverse && a.fc_bits == 0)
+      throw std::runtime_error("search_knn: reverse_cand needs ef_search below 1024 and fewer than 2^28 points");
     // with the keys in registers the queue's LDS share doubles as result buffer (lcap entries,
     // then lcap label slots) and as the replay heap (ef + 1 entries)
     const int floor_entries = ns > 0 ? std::max(ef + 1, 2 * a.lcap) : std::max(k, 64);
@@ -541,6 +545,7 @@ class Engine {
     a.nn_num0 = (int)(host.max_m0 * opt.heuristic_coef);
     a.nn_numU = (int)(host.max_m * opt.heuristic_coef);
     a.save_remains = opt.save_remains ? 1 : 0;
+    a.reverse = opt.reverse_cand ? 1 : 0;
     a.own_cap0 = own_links0 > 0 ? std::min(own_links0, host.max_m0) : host.max_m0;
     a.sel0_ids = d_sel0_ids.p; a.sel0_keys = d_sel0_keys.p; a.sel0_cnt = d_sel0_cnt.p;
     a.selU_ids = d_selU_ids.p; a.selU_keys = d_selU_keys.p; a.selU_cnt = d_selU_cnt.p;
@@ -555,6 +560,8 @@ class Engine {
                    (QR == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
     a.fc_bits = NS > 0 ? auto_fc_bits(efc) : 0;
     const bool sorted_set = NS > 0 && a.fc_bits > 0;  // then neither queue nor literal cache is needed
+    if (a.reverse && !sorted_set)
+      throw std::runtime_error("build_graph: reverse_cand needs ef_construction below 1024 and fewer than 2^28 points");
     a.cand_lds = sorted_set ? 0 : auto_cand_lds(efc, NS, 64, fixed);
     a.vc_bits = sorted_set ? 0 : auto_vc_bits();
     const LdsPlan lp1 = plan_lds(QR, Dp, sorted_set ? -1 : efc, a.cand_lds, a.lcap, efc, m_max, a.vc_bits, a.fc_bits);

@@ -60,12 +60,14 @@ struct SearchArgs {
   int vc_bits;  // log2 entries of the LDS visited cache of the literal search, 0 = none
   int fc_bits;  // log2 sets (two tags each) of the LDS visited filter of the sorted-set search, 0 = that search is off
   int fast_path;  // 0 = literal queues only (exact evaluation counters)
+  int reverse;    // expand the farthest waiting candidate (reverse_cand); sorted-set pass only
 };
 
 struct BuildArgs {
   int begin, count;        // batch = nodes begin .. begin+count-1
   int cur_ep, cur_max;     // entry point and top level of the graph before this batch (cur_max < 0: empty)
   int efc, nn_num0, nn_numU, save_remains;
+  int reverse;   // expand the farthest waiting candidate (reverse_cand)
   int own_cap0;  // how many links a new node may choose for itself on level 0 (<= max_m0)
   uint32_t* sel0_ids;  // count x max_m0: level-0 selections of the batch
   float* sel0_keys;
@@ -184,7 +186,7 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) s
     wave_sync();
     // (the flag is made wavefront-uniform explicitly and both outcomes are plain branches)
     const bool gave_up =
-        __builtin_amdgcn_readfirstlane((int)search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane)) != 0;
+        __builtin_amdgcn_readfirstlane((int)search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0)) != 0;
     if (gave_up) {
       if (lane == 0) {
         const int slot = atomicAdd(a.repeats, 1);
@@ -513,7 +515,7 @@ __global__ void __launch_bounds__(64) build_search_kernel(DevIndex ix, BuildArgs
           wave_sync();
           Frontier<NS> fr;
           frontier_init<NS>(fr, a.efc, lane);
-          search_level_fast<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, fr, 1, lane);
+          search_level_fast<DT, QR, NS, true>(ix, qv, level, a.efc, s, st, fr, 1, lane, a.reverse != 0);
           T = st.top_size;
           wave_sync();
           frontier_dump<NS>(fr, a.efc, T, sid, skey, lane);

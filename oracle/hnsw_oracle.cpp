@@ -38,6 +38,12 @@
 //                           0 returns the exact top-k), hand-walked tiny graphs
 //                           and invariants; bit-parity with a *real* hnswlib
 //                           binary is PARITY UNPINNED (not available offline).
+//   search_layer_far ...... (reverse_cand, cpp/include/cuda_utils_kernels.cuh:104-151)
+//                           pinned by a plain-Python statement of the same rule
+//                           incl. hop and evaluation counts, and by brute force
+//                           (ef >= N); against the CUDA reference itself PARITY
+//                           UNPINNED: it cannot run here and leaves the order
+//                           among equal distances to its warp reduction.
 //   file format ........... pinned by closed-form byte layout fixtures
 //   build ................. quality only (recall vs brute force, graph
 //                           invariants); PARITY UNPINNED against real hnswlib.
@@ -325,6 +331,58 @@ static MaxQueue search_layer(const Index& ix, const float* q, uint32_t ep, float
   return top;
 }
 
+// The reference's reverse_cand search (cuda_search_kernels.cuh:99-164 with GetCand(..., reverse = true),
+// cuda_utils_kernels.cuh:104-151): the result set of at most ef entries is also the candidate set; the
+// FARTHEST entry not yet expanded is expanded next, until none is left.  Not an hnswlib search.  The
+// reference leaves the order among equal distances to its warp reduction; here equal keys keep their
+// order of arrival (a stable sorted insert), the entry evicted from a full set is the last one, and the
+// result is the first k entries in that order.  Returns the set, ascending.
+struct SetEntry { float key; uint32_t id; bool expanded; };
+static std::vector<SetEntry> search_layer_far(const Index& ix, const float* q, uint32_t ep, float dep, int level, size_t ef,
+                                              Visited& vis, Counters* c) {
+  std::vector<SetEntry> set;
+  set.push_back({dep, ep, false});
+  vis.test_and_set(ep);
+  for (;;) {
+    int pick = -1;
+    for (int i = (int)set.size() - 1; i >= 0; --i) if (!set[i].expanded) { pick = i; break; }
+    if (pick < 0) break;
+    set[pick].expanded = true;
+    if (c) c->n_hops++;
+    const uint32_t* l = ix.list(set[pick].id, level);
+    uint32_t cnt = l[0];
+    for (uint32_t j = 0; j < cnt; ++j) {
+      uint32_t n = l[1 + j];
+      if (vis.test_and_set(n)) continue;
+      float d = canon_dist(q, ix.vec(n), ix.D, ix.dist_type);
+      if (c) c->n_dist++;
+      if (set.size() < ef || set.back().key > d) {
+        size_t pos = set.size();
+        while (pos > 0 && set[pos - 1].key > d) --pos;   // after every entry with key <= d
+        set.insert(set.begin() + pos, {d, n, false});
+        if (set.size() > ef) set.pop_back();
+      }
+    }
+  }
+  return set;
+}
+static int search_one_far(const Index& ix, const float* q, int k, int ef, Visited& vis, Counters* c,
+                          int* out_ids, float* out_d, int convention) {
+  if (ix.N == 0) return 0;
+  uint32_t cur = ix.enterpoint;
+  float dcur = canon_dist(q, ix.vec(cur), ix.D, ix.dist_type);
+  for (int level = ix.maxlevel; level > 0; --level) descend_level(ix, q, level, cur, dcur, c);
+  vis.reset(ix.N);
+  if (c) c->n_dist++;
+  std::vector<SetEntry> set = search_layer_far(ix, q, cur, dcur, 0, (size_t)std::max(ef, k), vis, c);
+  int found = (int)std::min<size_t>(set.size(), (size_t)k);
+  for (int i = 0; i < found; ++i) {
+    out_ids[i] = (int)ix.labels[set[i].id];
+    out_d[i] = convention == 1 ? api_dist(q, ix.vec(set[i].id), ix.D, ix.dist_type) : set[i].key;
+  }
+  return found;
+}
+
 // hnswlib searchKnn restated; results ascending by (distance, label) as the hnswlib python binding emits them.
 static int search_one(const Index& ix, const float* q, int k, int ef, Visited& vis, Counters* c,
                       int* out_ids, float* out_d, int convention) {
@@ -595,6 +653,25 @@ void orc_search(void* h, const float* q, int nq, int k, int ef, int* ids, float*
       if (counters) {
         long long* o = counters + (size_t)i * 5;
         o[0] = c.n_dist; o[1] = c.n_hops; o[2] = c.n_dist_upper; o[3] = c.n_sweeps_upper; o[4] = c.max_cand;
+      }
+    }
+  }
+}
+
+// the same for the reverse_cand search (farthest waiting entry first)
+void orc_search_far(void* h, const float* q, int nq, int k, int ef, int* ids, float* dists, int* found, long long* counters,
+                    int threads, int convention) {
+  const Index& ix = *static_cast<Index*>(h);
+#pragma omp parallel num_threads(threads > 0 ? threads : 1)
+  {
+    Visited vis;
+#pragma omp for schedule(dynamic, 16)
+    for (int i = 0; i < nq; ++i) {
+      Counters c;
+      found[i] = search_one_far(ix, q + (size_t)i * ix.D, k, ef, vis, &c, ids + (size_t)i * k, dists + (size_t)i * k, convention);
+      if (counters) {
+        long long* o = counters + (size_t)i * 5;
+        o[0] = c.n_dist; o[1] = c.n_hops; o[2] = c.n_dist_upper; o[3] = c.n_sweeps_upper; o[4] = 0;
       }
     }
   }

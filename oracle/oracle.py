@@ -71,6 +71,7 @@ def lib():
     l.orc_search.argtypes = [
         ctypes.c_void_p, _c_float_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _c_int_p, _c_float_p, _c_int_p, _c_ll_p, ctypes.c_int, ctypes.c_int]
+    l.orc_search_far.argtypes = l.orc_search.argtypes
     l.orc_descend.argtypes = [ctypes.c_void_p, _c_float_p, ctypes.c_int,
                               _c_int_p]
     l.orc_select.argtypes = [ctypes.c_void_p, _c_uint_p, _c_float_p,
@@ -229,7 +230,7 @@ class OracleIndex:
     return out[:n].copy()
 
   def search(self, queries, topk, ef_search, threads=None, convention="api",
-             counters=False):
+             counters=False, reverse_cand=False):
     """Returns (ids, distances, found[, counters]); rows ascending by
     (distance, label); entries beyond found[i] are undefined.
     counters columns: n_dist, n_hops, n_dist_upper, n_sweeps_upper, max_cand."""
@@ -241,7 +242,8 @@ class OracleIndex:
     dists = np.full((nq, topk), np.inf, dtype=np.float32)
     found = np.zeros(nq, dtype=np.int32)
     cnt = np.zeros((nq, 5), dtype=np.int64)
-    self._l.orc_search(self._h, _p(queries, _c_float_p), nq, topk, ef_search,
+    fn = self._l.orc_search_far if reverse_cand else self._l.orc_search
+    fn(self._h, _p(queries, _c_float_p), nq, topk, ef_search,
                        _p(ids, _c_int_p), _p(dists, _c_float_p),
                        _p(found, _c_int_p), _p(cnt, _c_ll_p),
                        threads or host_threads(),

@@ -131,3 +131,25 @@ def test_python_api_end_to_end(oracle, tmp_path):
   assert (one[0][0] == nns[0]).all()
   with pytest.raises(RuntimeError, match="dimension"):
     h2.search_knn(np.zeros((2, 7), np.float32), 1, 1)
+
+
+def test_build_with_reverse_cand(oracle, tmp_path):
+  """reverse_cand in the build (README of the reference: slower, better quality): the graph is
+  valid and at least as good as the plain build on the same data."""
+  n, d = 20000, 50
+  x = gauss_mixture(n, d, centres=200, seed=61)
+  q = gauss_mixture(300, d, centres=200, seed=62)
+  mult = 1.0 / np.log(12)
+  levels = _levels(n, mult, 63)
+  gt, _ = oracle.bruteforce(x, q, 10, "dot")
+  rec = {}
+  for rev in (False, True):
+    e = _build(tmp_path, x, levels, dist_type="dot", max_m=12, max_m0=24, ef_construction=60, heuristic_coef=0.0,
+               reverse_cand=rev)
+    p = str(tmp_path / ("rev%d.idx" % rev))
+    e.save_index(p)
+    ix = oracle.OracleIndex("dot").load(p)
+    assert ix.validate() == 0
+    ids, _, _ = ix.search(q, 10, 100)         # plain hnswlib search on both graphs
+    rec[rev] = recall(ids, gt)
+  assert rec[True] >= rec[False] - 0.01 and rec[True] >= 0.8, rec

@@ -243,3 +243,32 @@ def test_errors(tmp_path):
     e.search_knn(np.zeros((1, 4), np.float32), 1, 1)
   with pytest.raises(RuntimeError, match="set_random_levels first"):
     e.build_graph()
+
+
+@pytest.mark.parametrize("name,n,d,dist,max_m,max_m0,kind", [CASES[0], CASES[2], CASES[4], CASES[6]],
+                         ids=[CASES[i][0] for i in (0, 2, 4, 6)])
+def test_reverse_cand_search_parity(oracle, tmp_path, name, n, d, dist, max_m, max_m0, kind):
+  """The reference's reverse_cand option (the farthest waiting candidate is expanded first)
+  against the oracle's statement of it: ids, distances, found counts and expansion counters
+  identical, ties included (equal keys keep their order of arrival on both sides)."""
+  x = _data(kind, n, d, 1)
+  q = _data(kind, 120, d, 2)
+  mult = 1.0 / np.log(max_m)
+  ix = oracle.OracleIndex(dist).build(x, _levels(n, mult, 3), max_m, max_m0, 60, mult)
+  p = str(tmp_path / "i.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=max_m0, reverse_cand=True)
+  e.load_index(p)
+  for k, ef in ((10, 300), (1, 1), (10, 10), (100, 120), (10, 400), (50, 1023)):
+    o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True, reverse_cand=True)
+    g_ids, g_d, g_f = e.search_knn(q, k, ef)
+    assert (g_f == o_f).all()
+    for r in range(q.shape[0]):
+      f = o_f[r]
+      assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d k %d ef %d" % (r, k, ef)
+      assert (g_d[r, :f] == o_d[r, :f]).all()
+    d_ids, d_d, d_f, stats = _device_search(e, q, k, ef)
+    assert (d_ids == g_ids).all() and (stats[:, 1:] == o_cnt[:, 1:4]).all() and (stats[:, 0] >= o_cnt[:, 0]).all()
+    assert e.last_search_repeats == 0
+  with pytest.raises(RuntimeError, match="reverse_cand"):
+    e.search_knn(q, 10, 2000)

@@ -189,3 +189,58 @@ def test_tie_rich_search_matches_literal_model(oracle, seed):
     want = _model_search(x, links0, q[qi], k, ef)
     assert [i for _, i in want] == list(ids[qi, :found[qi]])
     assert [dd for dd, _ in want] == [float(v) for v in dists[qi, :found[qi]]]
+
+
+# ---- the reverse_cand search (farthest waiting entry first; cuda_utils_kernels.cuh:104-151) ----
+
+def _far_model(x, rows, q, ep, k, ef, dist):
+  """Plain-Python statement of the same search on a level-0-only index: a list kept sorted by
+  a stable insert, the last entry not yet expanded goes next, a full list drops its last."""
+  import bisect
+  keys, ids, done = [dist(q, x[ep])], [ep], [False]
+  seen = {ep}
+  hops = 0
+  while True:
+    pick = next((i for i in range(len(ids) - 1, -1, -1) if not done[i]), -1)
+    if pick < 0:
+      break
+    done[pick] = True
+    hops += 1
+    for nb in rows[ids[pick]]:
+      if nb in seen:
+        continue
+      seen.add(nb)
+      d = dist(q, x[nb])
+      if len(ids) < ef or keys[-1] > d:
+        pos = bisect.bisect_right(keys, d)
+        keys.insert(pos, d); ids.insert(pos, nb); done.insert(pos, False)
+        if len(ids) > ef:
+          keys.pop(); ids.pop(); done.pop()
+  return ids[:k], keys[:k], hops, len(seen)
+
+
+@pytest.mark.parametrize("kind", ["gauss", "tiny_int"])
+def test_reverse_cand_search_matches_plain_model(oracle, kind):
+  n, d = 400, 6
+  x = gauss_mixture(n, d, seed=31, normalise=False) if kind == "gauss" else integer_vectors(n, d, seed=31, hi=4)
+  q = gauss_mixture(25, d, seed=32, normalise=False) if kind == "gauss" else integer_vectors(25, d, seed=32, hi=4)
+  links0 = ring_graph(n, 6)
+  rows = [list(r[1:1 + r[0]]) for r in links0]
+  ix = flat_index(oracle, x, links0, "l2", 6)
+  dist = lambda a, b: oracle.distance(a, b, "l2")
+  for k, ef in ((5, 5), (10, 40), (3, 17)):
+    ids, dists, found, cnt = ix.search(q, k, ef, convention="hnswlib", counters=True, reverse_cand=True)
+    for r in range(q.shape[0]):
+      m_ids, m_keys, hops, seen = _far_model(x, rows, q[r], 0, k, ef, dist)
+      assert list(ids[r, :found[r]]) == m_ids and list(dists[r, :found[r]]) == m_keys
+      assert cnt[r, 1] == hops and cnt[r, 0] == seen
+
+
+def test_reverse_cand_search_with_ef_ge_n_is_brute_force(oracle):
+  n, d, k = 300, 17, 10
+  x = gauss_mixture(n, d, seed=5)
+  q = gauss_mixture(20, d, seed=6)
+  ix = flat_index(oracle, x, ring_graph(n, 8), "dot", 8)
+  ids, dists, found = ix.search(q, k, n, convention="hnswlib", reverse_cand=True)
+  bf_ids, bf_d = oracle.bruteforce(x, q, k, "dot")
+  assert (found == k).all() and (ids == bf_ids).all() and (dists == bf_d).all()
