@@ -679,6 +679,53 @@ __device__ __forceinline__ int frontier_take(Frontier<NS>& f, int lane, bool far
   for (int j = 0; j < N; ++j) f.v[j] = (lane == L && f.v[j] == id) ? (id | kExpanded) : f.v[j];
   return (int)id;
 }
+// key of the entry with this id (which is in the set)
+template <int NS>
+__device__ __forceinline__ float frontier_key_of(const Frontier<NS>& f, uint32_t id) {
+  constexpr int N = NS > 0 ? NS : 1;
+  float kf = 0.f;
+  bool hit = false;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const bool h = (f.v[j] & ~kExpanded) == id;
+    kf = h ? f.k[j] : kf;
+    hit = hit || h;
+  }
+  const unsigned long long mask = __ballot(hit);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, kf), __builtin_ctzll(mask | (1ull << 63))));
+}
+// is there an entry not yet expanded with exactly this key?
+template <int NS>
+__device__ __forceinline__ bool frontier_open_key(const Frontier<NS>& f, float key) {
+  constexpr int N = NS > 0 ? NS : 1;
+  bool hit = false;
+#pragma unroll
+  for (int j = 0; j < N; ++j) hit = hit || ((f.v[j] & kExpanded) == 0u && f.k[j] == key);
+  return __ballot(hit) != 0ull;
+}
+// do the two largest keys of a full set coincide?
+template <int NS>
+__device__ __forceinline__ bool frontier_max_twice(const Frontier<NS>& f) {
+  constexpr int N = NS > 0 ? NS : 1;
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f.k[N - 1]), 63));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f.k[N > 1 ? N - 2 : 0]), 63));
+  return a == b;
+}
+// do two neighbouring keys coincide among sorted positions p, p+1 with p < upto and p+1 < count?
+template <int NS>
+__device__ __forceinline__ bool frontier_tie_within(const Frontier<NS>& f, int ef, int upto, int count, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+  const float next_first = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, f.k[0]), 0x130, 0xF, 0xF, false));  // wave_shl:1
+  bool hit = false;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const int pos = lane * N + j - (64 * N - ef);
+    const float nxt = j + 1 < N ? f.k[j + 1 < N ? j + 1 : 0] : next_first;
+    hit = hit || (pos >= 0 && pos < upto && pos + 1 < count && f.k[j] == nxt);
+  }
+  return __ballot(hit) != 0ull;
+}
 // writes the sorted entries [0, count) to out_id / out_key (LDS)
 template <int NS>
 __device__ __forceinline__ void frontier_dump(const Frontier<NS>& f, int ef, int count, uint32_t* out_id, float* out_key,
@@ -736,21 +783,38 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
   }
 }
 
-// Best-first search of one level on the sorted set (needs the LDS tag cache).  On entry
-// s.nbuf[0..n_seed) holds the seeds, already entered into the filter.  Returns true as soon
-// as two equal keys meet in the set (BUILD: never; the search goes on).  Nearly all such
-// pairs are two waiting candidates, whose order of expansion is the heap's choice, so giving
-// up at once wastes the least work.  On a false return fr holds the result: st.top_size
-// entries, ascending, all keys distinct.  st.n_dist counts the evaluations performed,
-// repeated ones included.  far: expand the farthest waiting entry instead of the closest (the
-// reference's reverse_cand); that is no hnswlib search any more, equal keys simply keep their
-// order of arrival and the query is never given up.
+// Best-first search of one level on the sorted set (needs the LDS tag filter).  On entry
+// s.nbuf[0..n_seed) holds the seeds, already entered into the filter.  Returns 0: fr holds the
+// result (st.top_size entries, ascending), all keys were distinct; 2: the same, but equal keys
+// met on the way (the caller has to look at the cut at k); 1: given up — the outcome would
+// depend on how hnswlib's heaps lay equal keys out.  st.n_dist counts the evaluations
+// performed, repeated ones included.
+//
+// When do equal keys matter?  (a) Several waiting candidates share the smallest key d: hnswlib
+// expands them in its heap's order.  If none of their expansions produces a key below d the
+// order is immaterial — every node evaluated on the way is evaluated once whichever member
+// meets it first, a key below d would be accepted under any order (d is within the bound), so
+// none exists under any order, the whole group is expanded back to back and the set afterwards
+// is the ef smallest of old set and offers either way.  A key below d during the group gives
+// the query up.  (b) An eviction finds equal largest keys: which one leaves is the heap's
+// choice, and the one that leaves stays a live candidate of hnswlib as long as that key is
+// within the bound.  The search goes on, but gives up if it comes to expand an entry with such
+// a key, or ends while such a key is still within the bound.  (c) Equal keys among the k best
+// or across the cut: the caller's check.
+// far: expand the farthest waiting entry instead of the closest (the reference's
+// reverse_cand); that is no hnswlib search any more, equal keys simply keep their order of
+// arrival and nothing is ever given up.  BUILD likewise never gives up.
 template <int DT, int QR, int NS, bool BUILD>
-__device__ __forceinline__ bool search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
+__device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
                                                   SearchState& st, Frontier<NS>& fr, int n_seed, int lane,
                                                   bool far = false) {
   const int S = row_stride(ix, level);
   int n = n_seed;
+  const bool exact = !BUILD && !far;  // the outcome has to be hnswlib's
+  bool have_tie = false;              // equal keys have met in the set
+  bool in_group = false;              // the entries being expanded share one key with others still waiting
+  float group_key = 0.f;
+  float ek_min = INFINITY;            // smallest key at which an eviction had equal largest keys to choose from
   while (true) {
     if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
     st.n_dist += n;
@@ -766,9 +830,15 @@ __device__ __forceinline__ bool search_level_fast(const DevIndex& ix, const QVec
         const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
         const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
         if (!(st.n_acc < ef || st.lower > key)) continue;
+        // an eviction out of several equal largest keys: the heap's choice decides which of
+        // them stays in the result set, and the other one stays a live candidate of hnswlib
+        if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = fminf(ek_min, st.lower);
         const int r = frontier_insert<NS>(fr, key, id, lane);
         if (r == 2) continue;
-        if (!BUILD && !far && r == 1) return true;
+        have_tie = have_tie || r == 1;
+        // a closer candidate turning up while a group of equal keys is being expanded would be
+        // expanded before or after the rest of the group depending on the heap's order
+        if (exact && in_group && key < group_key) return 1;
         st.n_acc += 1;
         st.maxkey = fmaxf(st.maxkey, key);
         st.lower = st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey;  // hnswlib's lowerBound
@@ -776,13 +846,26 @@ __device__ __forceinline__ bool search_level_fast(const DevIndex& ix, const QVec
     }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     const int cid = frontier_take<NS>(fr, lane, far);
-    if (cid < 0) break;
+    if (cid < 0) {
+      // an entry evicted out of equal largest keys that are still within the bound is one
+      // hnswlib would go on to expand
+      if (exact && st.n_acc >= ef && st.lower >= ek_min) return 1;
+      break;
+    }
+    if (exact && have_tie) {
+      const float d = frontier_key_of<NS>(fr, (uint32_t)cid);
+      if (d >= ek_min) return 1;
+      if (!(in_group && d == group_key)) {
+        in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
+        group_key = d;
+      }
+    }
     st.n_hops += 1;
     wave_sync();
     n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
     wave_sync();
   }
-  return false;
+  return have_tie ? 2 : 0;
 }
 
 // Greedy descent through levels from_level .. to_level+1 (hnswlib searchKnn upper

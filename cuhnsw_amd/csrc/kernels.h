@@ -185,8 +185,12 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) s
     if (lane == 0) s.nbuf[0] = cur;
     wave_sync();
     // (the flag is made wavefront-uniform explicitly and both outcomes are plain branches)
-    const bool gave_up =
-        __builtin_amdgcn_readfirstlane((int)search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0)) != 0;
+    const int how =
+        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0));
+    const int T0 = st.top_size < a.k ? st.top_size : a.k;
+    // equal keys among the k best or across the cut: order and membership follow the
+    // (distance, label) rule and the result heap, which the literal search reproduces
+    const bool gave_up = how == 1 || (how == 2 && !a.reverse && frontier_tie_within<NS>(fr, a.ef, T0, st.top_size, lane));
     if (gave_up) {
       if (lane == 0) {
         const int slot = atomicAdd(a.repeats, 1);
