@@ -82,7 +82,8 @@ class Engine {
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
   int spin_limit_override = -1;  // polls a waiting literal wavefront may spend (-1 = automatic)
-  int side_per_cu = 4;         // its wavefronts per CU
+  int side_per_cu = 0;         // its wavefronts per CU (0 = from the share of queries the last search gave up)
+  double last_repeat_share = 0.0;         // its wavefronts per CU
   int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
@@ -370,10 +371,13 @@ class Engine {
       int slots = resident_slots(fast_kernel, fp.total);
       const bool side = concurrent_literal && max_slots_override <= 0;
       int side_slots = 0;
+      // few queries need the literal pass (0.4 % of the 1.18M-point set's): one wavefront per CU
+      // serves them without taking room from the first pass; more when the last search needed more
+      const int per_cu = side_per_cu > 0 ? side_per_cu : (last_repeat_share < 0.02 ? 1 : (last_repeat_share < 0.06 ? 2 : 4));
       if (side) {
-        side_slots = std::min(num_cus * side_per_cu, a.nq);
+        side_slots = std::min(num_cus * per_cu, a.nq);
         ensure_pool(std::max(side_slots, 1), glob_cap, 2 * glob_cap);
-        slots = std::max(num_cus, slots - num_cus * side_per_cu);  // leave the literal wavefronts their room
+        slots = std::max(num_cus, slots - num_cus * per_cu);  // leave the literal wavefronts their room
       }
       if (max_slots_override > 0) slots = max_slots_override;
       slots = std::max(1, std::min(slots, a.nq));
@@ -399,6 +403,7 @@ class Engine {
       HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
       HIP_CHECK(hipStreamSynchronize(stream));
       n_literal = last_repeats = ctl[32];
+      last_repeat_share = (double)n_literal / a.nq;
       // an index whose distances tie all the time (integer-valued data) sends most queries
       // through both passes: stop trying the sorted set on it
       if (a.nq >= 256 && (long long)n_literal * 3 > a.nq) fast_suspended = true;
@@ -771,7 +776,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
   else if (n == "concurrent_literal") e->impl.concurrent_literal = value != 0.0;
   else if (n == "literal_spin_limit") e->impl.spin_limit_override = (int)value;
-  else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(1, std::min(8, (int)value));
+  else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(0, std::min(8, (int)value));
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else return -1;
   return 0;
