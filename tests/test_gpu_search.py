@@ -272,3 +272,34 @@ def test_reverse_cand_search_parity(oracle, tmp_path, name, n, d, dist, max_m, m
     assert e.last_search_repeats == 0
   with pytest.raises(RuntimeError, match="reverse_cand"):
     e.search_knn(q, 10, 2000)
+
+
+@pytest.mark.parametrize("seed,d,hi", [(101, 12, 12), (102, 8, 40), (103, 24, 6), (104, 5, 200)])
+def test_followed_up_ties_match_the_oracle_on_quantised_data(oracle, tmp_path, seed, d, hi):
+  """Quantised data: equal distances everywhere, but most of them harmless.  The sorted-set
+  pass follows groups of equal keys up instead of giving every such query to the literal
+  queues; ids, distances and expansion counts must still be the oracle's for every query, at
+  many (k, ef) shapes, with and without labels that differ from the ids."""
+  n = 8000
+  x = integer_vectors(n, d, seed=seed, hi=hi)
+  q = integer_vectors(700, d, seed=seed + 50, hi=hi)
+  mult = 1 / np.log(8)
+  levels = _levels(n, mult, seed + 7)
+  ix = oracle.OracleIndex("l2").build(x, levels, 8, 16, 50, mult)
+  p = str(tmp_path / "qd.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
+  e.load_index(p)
+  e.set_tunable("fast_path", 2)
+  answered_by_first_pass = 0
+  for k, ef in ((10, 64), (10, 300), (1, 16), (100, 100), (32, 33), (5, 319), (10, 700)):
+    o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
+    g_ids, g_d, g_f, stats = _device_search(e, q, k, ef)
+    assert (g_f == o_f).all()
+    for r in range(q.shape[0]):
+      f = o_f[r]
+      assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d k %d ef %d" % (r, k, ef)
+      assert (g_d[r, :f] == o_d[r, :f]).all()
+    assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
+    answered_by_first_pass += q.shape[0] - e.last_search_repeats
+  assert answered_by_first_pass > 0

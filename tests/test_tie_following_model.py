@@ -1,0 +1,105 @@
+"""Pins the argument behind the sorted-set search's handling of equal keys (the rules in
+search_level_fast, cuhnsw_amd/csrc/device_core.h), on the CPU: a plain-Python statement of
+those rules is run on small random graphs whose integer coordinates make distances tie all
+the time, and whenever it does NOT give a query up, its answer — ids, distances and the number
+of expansions and evaluations — must be what the oracle's literal hnswlib search
+(two std::priority_queues) returns.  A rule that lets an order-dependent case through shows
+up here as a mismatch within a few thousand trials."""
+import numpy as np
+import pytest
+
+INF = float("inf")
+
+
+def sorted_set_search(keys_of, rows, ep, k, ef):
+  """Returns None when given up, else (ids, keys, hops, evaluations, met equal keys)."""
+  S = [[keys_of(ep), ep, False]]          # sorted by key, equal keys in order of arrival
+  seen = {ep}
+  have_tie = in_group = False
+  group_key = 0.0
+  ek_min = INF
+  hops = 0
+  offers = []
+  while True:
+    for key, node in offers:
+      full = len(S) >= ef
+      if full and not (S[-1][0] > key):
+        continue
+      if have_tie and full and S[-1][0] == S[-2][0]:
+        ek_min = min(ek_min, S[-1][0])        # eviction with equal largest keys to choose from
+      if any(e[0] == key for e in S):
+        have_tie = True
+      if in_group and key < group_key:
+        return None                           # a closer candidate inside a group of equal keys
+      pos = len(S)
+      while pos > 0 and S[pos - 1][0] > key:
+        pos -= 1
+      S.insert(pos, [key, node, False])
+      if len(S) > ef:
+        S.pop()
+    pick = next((i for i, e in enumerate(S) if not e[2]), -1)
+    if pick < 0:
+      if len(S) >= ef and S[-1][0] >= ek_min:
+        return None                           # an evicted twin is still a live candidate of hnswlib
+      break
+    d = S[pick][0]
+    if have_tie:
+      if d >= ek_min:
+        return None
+      if not (in_group and d == group_key):
+        in_group = any((not e[2]) and e[0] == d for i, e in enumerate(S) if i != pick)
+        group_key = d
+    S[pick][2] = True
+    hops += 1
+    offers = []
+    for nb in rows[S[pick][1]]:
+      if nb not in seen:
+        seen.add(nb)
+        offers.append((keys_of(nb), nb))
+  T = min(k, len(S))
+  if have_tie and any(S[p][0] == S[p + 1][0] for p in range(T) if p + 1 < len(S)):
+    return None                               # equal keys among the k best or across the cut
+  return [e[1] for e in S[:T]], [e[0] for e in S[:T]], hops, len(seen), have_tie
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_rules_never_let_an_order_dependent_case_through(oracle, seed):
+  rng = np.random.default_rng(1000 + seed)
+  answered = given_up = answered_with_ties = 0
+  for graph in range(60):
+    n = int(rng.integers(12, 60))
+    dim = int(rng.integers(1, 4))
+    hi = int(rng.integers(3, 30))
+    x = rng.integers(0, hi, (n, dim)).astype(np.float32)
+    deg = int(rng.integers(2, 7))
+    links0 = np.zeros((n, 1 + 8), np.uint32)
+    rows = []
+    for i in range(n):
+      others = [j for j in range(n) if j != i]
+      nb = list(rng.choice(others, size=min(deg, len(others)), replace=False))
+      nb.append((i + 1) % n)                  # a ring keeps everything reachable
+      nb = list(dict.fromkeys(int(v) for v in nb if v != i))[:8]
+      links0[i, 0] = len(nb)
+      links0[i, 1:1 + len(nb)] = nb
+      rows.append(nb)
+    ix = oracle.OracleIndex("l2").from_arrays(x, np.zeros(n, np.int32), links0, np.zeros(0, np.uint32),
+                                              max_m=4, max_m0=8, maxlevel=0, enterpoint=0)
+    q = rng.integers(0, hi, (24, dim)).astype(np.float32)
+    for k, ef in ((1, 1), (2, 3), (3, 5), (4, 4), (5, 8), (2, 12)):
+      ids, dists, found, cnt = ix.search(q, k, ef, convention="hnswlib", counters=True)
+      for r in range(q.shape[0]):
+        keys_of = lambda node, qq=q[r]: float(np.float32(((qq - x[node]) ** 2).sum()))
+        got = sorted_set_search(keys_of, rows, 0, k, ef)
+        if got is None:
+          given_up += 1
+          continue
+        answered += 1
+        m_ids, m_keys, hops, evals, tied = got
+        answered_with_ties += bool(tied)
+        f = found[r]
+        assert f == len(m_ids)
+        assert list(ids[r, :f]) == m_ids, (seed, graph, r, k, ef)
+        assert list(dists[r, :f]) == m_keys
+        assert cnt[r, 1] == hops and cnt[r, 0] == evals, (seed, graph, r, k, ef)
+  # both outcomes are exercised, and so are searches that met equal keys and were still answered
+  assert answered > 1000 and given_up > 100 and answered_with_ties > 300, (answered, given_up, answered_with_ties)
