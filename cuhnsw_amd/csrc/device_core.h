@@ -795,8 +795,11 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 // order is immaterial — every node evaluated on the way is evaluated once whichever member
 // meets it first, a key below d would be accepted under any order (d is within the bound), so
 // none exists under any order, the whole group is expanded back to back and the set afterwards
-// is the ef smallest of old set and offers either way.  A key below d during the group gives
-// the query up.  (b) An eviction finds equal largest keys: which one leaves is the heap's
+// is the ef smallest of old set and offers either way — up to entries whose key equals the
+// bound the set ends up with: whether such an offer is accepted or turned away, and which of
+// several such entries is evicted, does depend on the order.  So a key below d during the
+// group gives the query up, and so does a group during which an offer was turned away or an
+// entry evicted whose key equals the bound at the group's end.  (b) An eviction finds equal largest keys: which one leaves is the heap's
 // choice, and the one that leaves stays a live candidate of hnswlib as long as that key is
 // within the bound.  The search goes on, but gives up if it comes to expand an entry with such
 // a key, or ends while such a key is still within the bound.  (c) Equal keys among the k best
@@ -814,6 +817,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   bool have_tie = false;              // equal keys have met in the set
   bool in_group = false;              // the entries being expanded share one key with others still waiting
   float group_key = 0.f;
+  float group_edge = INFINITY;        // closest key turned away or evicted while the group is expanded
   float ek_min = INFINITY;            // smallest key at which an eviction had equal largest keys to choose from
   while (true) {
     if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
@@ -823,13 +827,19 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       const int mine = base + lane;
       const float my_key = mine < n ? s.dbuf[mine] : INFINITY;
       const uint32_t my_id = mine < n ? s.nbuf[mine] : 0u;
-      unsigned long long todo = __ballot(mine < n && (st.n_acc < ef || st.lower > my_key));
+      const bool pass = mine < n && (st.n_acc < ef || st.lower > my_key);
+      unsigned long long todo = __ballot(pass);
+      // offers turned away while a group of equal keys is being expanded: remember the closest
+      if (exact && in_group) group_edge = fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY));
       while (todo != 0ull) {
         const int j = __builtin_ctzll(todo);
         todo &= todo - 1ull;
         const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
         const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
-        if (!(st.n_acc < ef || st.lower > key)) continue;
+        if (!(st.n_acc < ef || st.lower > key)) {
+          if (exact && in_group) group_edge = fminf(group_edge, key);
+          continue;
+        }
         // an eviction out of several equal largest keys: the heap's choice decides which of
         // them stays in the result set, and the other one stays a live candidate of hnswlib
         if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = fminf(ek_min, st.lower);
@@ -839,6 +849,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
         // a closer candidate turning up while a group of equal keys is being expanded would be
         // expanded before or after the rest of the group depending on the heap's order
         if (exact && in_group && key < group_key) return 1;
+        if (exact && in_group && st.n_acc >= ef) group_edge = fminf(group_edge, st.lower);  // the entry this insert evicted
         st.n_acc += 1;
         st.maxkey = fmaxf(st.maxkey, key);
         st.lower = st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey;  // hnswlib's lowerBound
@@ -846,19 +857,28 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
     }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     const int cid = frontier_take<NS>(fr, lane, far);
+    if (exact && have_tie) {
+      const float d = cid >= 0 ? frontier_key_of<NS>(fr, (uint32_t)cid) : INFINITY;
+      if (in_group && d != group_key) {
+        // the group is through.  With another order of its members an offer or an entry whose
+        // key equals the bound reached now could have ended up on the other side of it.
+        if (st.n_acc >= ef && group_edge == st.lower) return 1;
+        in_group = false;
+      }
+      if (cid >= 0) {
+        if (d >= ek_min) return 1;
+        if (!in_group) {
+          in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
+          group_key = d;
+          group_edge = INFINITY;
+        }
+      }
+    }
     if (cid < 0) {
       // an entry evicted out of equal largest keys that are still within the bound is one
       // hnswlib would go on to expand
       if (exact && st.n_acc >= ef && st.lower >= ek_min) return 1;
       break;
-    }
-    if (exact && have_tie) {
-      const float d = frontier_key_of<NS>(fr, (uint32_t)cid);
-      if (d >= ek_min) return 1;
-      if (!(in_group && d == group_key)) {
-        in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
-        group_key = d;
-      }
     }
     st.n_hops += 1;
     wave_sync();
