@@ -116,6 +116,12 @@ __device__ __forceinline__ float reduce16(float x) {
   x = x + dpp_move<0x140>(x);  // row_mirror
   return x;
 }
+// Tells the compiler that a value is the same in all lanes (it is then kept in a scalar register
+// and branches on it are scalar branches instead of exec-mask juggling).
+__device__ __forceinline__ float uni(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+}
+__device__ __forceinline__ int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
 __device__ __forceinline__ float wave_min(float x) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) x = fminf(x, __shfl_xor(x, m, 64));
@@ -830,29 +836,29 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       const bool pass = mine < n && (st.n_acc < ef || st.lower > my_key);
       unsigned long long todo = __ballot(pass);
       // offers turned away while a group of equal keys is being expanded: remember the closest
-      if (exact && in_group) group_edge = fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY));
+      if (exact && in_group) group_edge = uni(fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY)));
       while (todo != 0ull) {
         const int j = __builtin_ctzll(todo);
         todo &= todo - 1ull;
         const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
         const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
         if (!(st.n_acc < ef || st.lower > key)) {
-          if (exact && in_group) group_edge = fminf(group_edge, key);
+          if (exact && in_group) group_edge = uni(fminf(group_edge, key));
           continue;
         }
         // an eviction out of several equal largest keys: the heap's choice decides which of
         // them stays in the result set, and the other one stays a live candidate of hnswlib
-        if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = fminf(ek_min, st.lower);
+        if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = uni(fminf(ek_min, st.lower));
         const int r = frontier_insert<NS>(fr, key, id, lane);
         if (r == 2) continue;
         have_tie = have_tie || r == 1;
         // a closer candidate turning up while a group of equal keys is being expanded would be
         // expanded before or after the rest of the group depending on the heap's order
         if (exact && in_group && key < group_key) return 1;
-        if (exact && in_group && st.n_acc >= ef) group_edge = fminf(group_edge, st.lower);  // the entry this insert evicted
-        st.n_acc += 1;
-        st.maxkey = fmaxf(st.maxkey, key);
-        st.lower = st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey;  // hnswlib's lowerBound
+        if (exact && in_group && st.n_acc >= ef) group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
+        st.n_acc = uni(st.n_acc + 1);
+        st.maxkey = uni(fmaxf(st.maxkey, key));
+        st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
       }
     }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;

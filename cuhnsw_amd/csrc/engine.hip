@@ -573,7 +573,8 @@ class Engine {
     const LdsPlan lp3 = plan_lds(QR, Dp, s_max + cap_in, 0, a.lcap, s_max + cap_in, m_max);
     const int slots1 = resident_slots(k_search, lp1.total);
     const int slots3 = resident_slots(k_reverse, lp3.total);
-    ensure_pool(slots1, glob_cap, 2 * glob_cap);
+    // the sorted-set search needs no per-wavefront global memory (no bitmap, no undo list, no log)
+    if (!sorted_set) ensure_pool(slots1, glob_cap, 2 * glob_cap);
     a.pool = pool;
 
     // Nodes go in by ascending id, as hnswlib inserts them.  The graph a batch sees is the
