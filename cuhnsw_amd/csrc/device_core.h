@@ -766,7 +766,8 @@ __device__ __forceinline__ int visit_lossy(const uint32_t* row, int S, Scratch& 
   uint32_t* sets = reinterpret_cast<uint32_t*>(s.vcache);
   const uint32_t mask_bits = (1u << s.vc_bits) - 1u;
   for (int base = 0; base < S; base += 64) {
-    const uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
+    const uint32_t got = row[base + lane < S ? base + lane : 0];  // unconditional load, then a select
+    const uint32_t id = (base + lane < S) ? got : kEmpty;
     bool ask = id != kEmpty;
     if (ask) {
       const uint32_t slot = id & mask_bits;
@@ -831,8 +832,10 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
     wave_sync();
     for (int base = 0; base < n; base += 64) {
       const int mine = base + lane;
-      const float my_key = mine < n ? s.dbuf[mine] : INFINITY;
-      const uint32_t my_id = mine < n ? s.nbuf[mine] : 0u;
+      // unconditional LDS reads at a clamped index, then a select: no exec-mask branches
+      const int at = mine < n ? mine : 0;
+      const float my_key = mine < n ? s.dbuf[at] : INFINITY;
+      const uint32_t my_id = s.nbuf[at];
       const bool pass = mine < n && (st.n_acc < ef || st.lower > my_key);
       unsigned long long todo = __ballot(pass);
       // offers turned away while a group of equal keys is being expanded: remember the closest
@@ -926,8 +929,8 @@ __device__ __forceinline__ void descend(const DevIndex& ix, const QVec<QR>& qv, 
         }
       }
       if (bidx >= 0 && best < dcur) {
-        dcur = best;
-        cur = s.nbuf[bidx];
+        dcur = uni(best);
+        cur = (uint32_t)uni((int)s.nbuf[bidx]);
         changed = true;
       }
       wave_sync();
