@@ -286,7 +286,7 @@ class Engine {
 
   // slots of sorted result keys per lane: the result set lives in registers while
   // ef < 64 * NS; 0 selects the literal LDS heap for larger ef
-  static int key_slots(int ef) { return ef < 320 ? 5 : (ef <= 512 ? 8 : (ef < 1024 ? 16 : 0)); }
+  static int key_slots(int ef) { return ef <= 128 ? 2 : (ef < 320 ? 5 : (ef <= 512 ? 8 : (ef < 1024 ? 16 : 0))); }
 
   // LDS entries of the candidate queue.  With the result keys in registers the queue is the
   // only large LDS user: 2*ef entries hold it in nearly every query (the rest spills to the
@@ -444,6 +444,7 @@ class Engine {
   template <int DT, int QR>
   void launch_search_ns(int ns, const DevIndex& ix, SearchArgs& a, float* ms) {
     switch (ns) {
+      case 2: launch_search<DT, QR, 2>(ix, a, search_slots, ms); break;
       case 5: launch_search<DT, QR, 5>(ix, a, search_slots, ms); break;
       case 8: launch_search<DT, QR, 8>(ix, a, search_slots, ms); break;
       case 16: launch_search<DT, QR, 16>(ix, a, search_slots, ms); break;
@@ -622,6 +623,7 @@ class Engine {
   template <int DT, int QR>
   void build_ns(int ns) {
     switch (ns) {
+      case 2: build_levels<DT, QR, 2>(); break;
       case 5: build_levels<DT, QR, 5>(); break;
       case 8: build_levels<DT, QR, 8>(); break;
       case 16: build_levels<DT, QR, 16>(); break;

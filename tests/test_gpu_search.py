@@ -100,8 +100,9 @@ def test_search_parity_on_oracle_built_index(oracle, tmp_path, name, n, d, dist,
   e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=max_m0)
   e.load_index(p)
   assert (e.num_data, e.num_dims, e.max_level, e.enter_point) == (n, d, ix.maxlevel, ix.enterpoint)
-  # ef < 320: result keys in 5 registers per lane; <= 512: 8; < 1024: 16; beyond: literal LDS heap
-  for k, ef in ((10, 300), (1, 1), (10, 10), (100, 64), (100, 120), (7, 33), (10, 400), (100, 512), (10, 513),
+  # ef <= 128: result keys in 2 registers per lane; < 320: 5; <= 512: 8; < 1024: 16; beyond: literal LDS heap
+  for k, ef in ((10, 300), (1, 1), (10, 10), (100, 64), (100, 120), (7, 33), (128, 128), (10, 129), (10, 400),
+                (100, 512), (10, 513),
                 (50, 1023), (10, 1100)):
     _check_parity(oracle, ix, e, q, k, ef)
 
