@@ -38,6 +38,7 @@ def main():
   ap.add_argument("--n", type=int, default=None, help="shrink the data set (debugging)")
   ap.add_argument("--nq", type=int, default=None)
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--ef", type=int, default=None, help="ef_search (default: the configuration's headline value)")
   ap.add_argument("--copy-calibration", action="store_true",
                   help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   args = ap.parse_args()
@@ -57,6 +58,8 @@ def main():
   o = dict(spec["opt"])
   n, d = data.shape
   nq, k, ef = queries.shape[0], spec["topk"], spec["ef"][-1] if args.workload != "C2" else 300
+  if args.ef:
+    ef = max(args.ef, k)
   mult = o.get("level_mult") or 1.0 / np.log(o["max_m"])
   levels = datasets.random_levels(n, mult)
   gen_s = time.time() - t0
