@@ -218,7 +218,9 @@ def main():
       o_ids, o_d, o_f = ix.search(queries[:n_s], k, ef, threads=cores)
       passes += 1
     cpu_search_s = (time.perf_counter() - t0) / passes
-    mism = int((o_ids != ids[:n_s]).any(axis=1).sum())
+    bad_rows = (o_ids != ids[:n_s]).any(axis=1)
+    mism = int(bad_rows.sum())
+    tied = ix.meets_ties(queries[:n_s], ef, threads=cores)   # queries whose search meets equal distances
     n_b = min(n, 400000)
     t0 = time.perf_counter()
     orc.OracleIndex(o["dist_type"]).build(data[:n_b], levels[:n_b], o["max_m"], o["max_m0"], o["ef_construction"],
@@ -232,7 +234,10 @@ def main():
         "build_points_per_s": n_b / cpu_build_s,
         "gpu_build_points_per_s": n / build_s,
     }
-    out["parity"] = {"queries_checked": n_s, "rows_with_id_mismatch_vs_oracle": mism}
+    out["parity"] = {"queries_checked": n_s, "rows_with_id_mismatch_vs_oracle": mism,
+                     "queries_meeting_equal_distances": int(tied.sum()),
+                     "id_mismatches_among_them": int((bad_rows & tied).sum()),
+                     "id_mismatches_among_the_rest": int((bad_rows & ~tied).sum())}
   print(json.dumps(out))
 
 

@@ -62,6 +62,7 @@
 #include <mutex>
 #include <queue>
 #include <string>
+#include <set>
 #include <vector>
 #ifdef _OPENMP
 #include <omp.h>
@@ -383,6 +384,43 @@ static int search_one_far(const Index& ix, const float* q, int k, int ef, Visite
   return found;
 }
 
+// The same search, only to learn whether the query meets equal distances on its way: true if a key
+// accepted into the result set equals a key that is in the result set at that moment.  Those are the
+// queries whose answer can depend on how the priority queues lay equal keys out (the reference's README
+// claims id-equality with hnswlib, README.md:112-113, which its single-heap kernel can only keep for the
+// others).
+static bool search_meets_ties(const Index& ix, const float* q, uint32_t ep, float dep, size_t ef, Visited& vis) {
+  MaxQueue top, cand;
+  std::multiset<float> keys;
+  bool met = false;
+  float lowerBound = dep;
+  top.emplace(dep, ep);
+  cand.emplace(-dep, ep);
+  keys.insert(dep);
+  vis.test_and_set(ep);
+  while (!cand.empty()) {
+    DistId cur = cand.top();
+    if ((-cur.first) > lowerBound) break;
+    cand.pop();
+    const uint32_t* l = ix.list(cur.second, 0);
+    uint32_t cnt = l[0];
+    for (uint32_t j = 0; j < cnt; ++j) {
+      uint32_t n = l[1 + j];
+      if (vis.test_and_set(n)) continue;
+      float d = canon_dist(q, ix.vec(n), ix.D, ix.dist_type);
+      if (top.size() < ef || lowerBound > d) {
+        if (keys.count(d)) met = true;
+        keys.insert(d);
+        cand.emplace(-d, n);
+        top.emplace(d, n);
+        if (top.size() > ef) { keys.erase(keys.find(top.top().first)); top.pop(); }
+        if (!top.empty()) lowerBound = top.top().first;
+      }
+    }
+  }
+  return met;
+}
+
 // hnswlib searchKnn restated; results ascending by (distance, label) as the hnswlib python binding emits them.
 static int search_one(const Index& ix, const float* q, int k, int ef, Visited& vis, Counters* c,
                       int* out_ids, float* out_d, int convention) {
@@ -654,6 +692,26 @@ void orc_search(void* h, const float* q, int nq, int k, int ef, int* ids, float*
         long long* o = counters + (size_t)i * 5;
         o[0] = c.n_dist; o[1] = c.n_hops; o[2] = c.n_dist_upper; o[3] = c.n_sweeps_upper; o[4] = c.max_cand;
       }
+    }
+  }
+}
+
+// per query: 1 if the hnswlib search meets equal distances in its result set, else 0
+void orc_search_meets_ties(void* h, const float* q, int nq, int ef, unsigned char* out, int threads) {
+  const Index& ix = *static_cast<Index*>(h);
+#pragma omp parallel num_threads(threads > 0 ? threads : 1)
+  {
+    Visited vis;
+#pragma omp for schedule(dynamic, 16)
+    for (int i = 0; i < nq; ++i) {
+      const float* qi = q + (size_t)i * ix.D;
+      out[i] = 0;
+      if (ix.N == 0) continue;
+      uint32_t cur = ix.enterpoint;
+      float dcur = canon_dist(qi, ix.vec(cur), ix.D, ix.dist_type);
+      for (int level = ix.maxlevel; level > 0; --level) descend_level(ix, qi, level, cur, dcur, nullptr);
+      vis.reset(ix.N);
+      out[i] = search_meets_ties(ix, qi, cur, dcur, (size_t)ef, vis) ? 1 : 0;
     }
   }
 }

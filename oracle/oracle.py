@@ -72,6 +72,8 @@ def lib():
         ctypes.c_void_p, _c_float_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _c_int_p, _c_float_p, _c_int_p, _c_ll_p, ctypes.c_int, ctypes.c_int]
     l.orc_search_far.argtypes = l.orc_search.argtypes
+    l.orc_search_meets_ties.argtypes = [ctypes.c_void_p, _c_float_p, ctypes.c_int, ctypes.c_int,
+                                        ctypes.POINTER(ctypes.c_ubyte), ctypes.c_int]
     l.orc_descend.argtypes = [ctypes.c_void_p, _c_float_p, ctypes.c_int,
                               _c_int_p]
     l.orc_select.argtypes = [ctypes.c_void_p, _c_uint_p, _c_float_p,
@@ -228,6 +230,14 @@ class OracleIndex:
                            _p(cand_dists, _c_float_p), cand_ids.shape[0], m,
                            _p(out, _c_uint_p))
     return out[:n].copy()
+
+  def meets_ties(self, queries, ef_search, threads=None):
+    """Per query: does the hnswlib search meet equal distances in its result set?"""
+    queries = _f32(queries)
+    out = np.zeros(queries.shape[0], dtype=np.uint8)
+    self._l.orc_search_meets_ties(self._h, _p(queries, _c_float_p), queries.shape[0], ef_search,
+                                  out.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), threads or host_threads())
+    return out.astype(bool)
 
   def search(self, queries, topk, ef_search, threads=None, convention="api",
              counters=False, reverse_cand=False):

@@ -244,3 +244,22 @@ def test_reverse_cand_search_with_ef_ge_n_is_brute_force(oracle):
   ids, dists, found = ix.search(q, k, n, convention="hnswlib", reverse_cand=True)
   bf_ids, bf_d = oracle.bruteforce(x, q, k, "dot")
   assert (found == k).all() and (ids == bf_ids).all() and (dists == bf_d).all()
+
+
+def test_meets_ties_flags_exactly_the_queries_with_equal_keys(oracle):
+  # tie-free data: nothing flagged; data on a coarse grid: everything flagged; and the flag
+  # agrees with a direct look at the distances of all nodes a full search (ef >= N) accepts
+  n, d = 300, 5
+  x = gauss_mixture(n, d, seed=41, normalise=False)
+  q = gauss_mixture(30, d, seed=42, normalise=False)
+  ix = flat_index(oracle, x, ring_graph(n, 8), "l2", 8)
+  assert not ix.meets_ties(q, n).any()
+  xi = integer_vectors(n, 2, seed=43, hi=3)
+  qi = integer_vectors(30, 2, seed=44, hi=3)
+  ixi = flat_index(oracle, xi, ring_graph(n, 8), "l2", 8)
+  assert ixi.meets_ties(qi, n).all()
+  # one duplicated point: only queries are flagged for which it matters, i.e. all (ef >= N
+  # accepts every node, the duplicate's key repeats)
+  xd = x.copy(); xd[17] = xd[200]
+  ixd = flat_index(oracle, xd, ring_graph(n, 8), "l2", 8)
+  assert ixd.meets_ties(q, n).all()
