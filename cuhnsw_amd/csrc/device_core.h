@@ -897,6 +897,87 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   return have_tie ? 2 : 0;
 }
 
+// hnswlib's level-0 search with the literal candidate queue (which alone decides the order of
+// expansion among equal keys) but with the sorted set with ids as result set and the LDS-only
+// visited filter of the sorted-set search: a neighbour the filter has forgotten is evaluated
+// again and then either found in the set by its id, or turned away by the accept rule as it
+// was (or would be) the first time — the candidate queue sees exactly hnswlib's sequence of
+// pushes and pops.  No bitmap, no atomics, nothing to undo.  Every accepted entry is also
+// logged (s.log) for the caller's replay of the result heap.  *ambiguous is set when an
+// eviction had equal largest keys to choose from: the set then holds the same keys as
+// hnswlib's result heap but possibly another of the twins.  st.n_dist counts the evaluations
+// performed, repeated ones included.  On entry s.nbuf[0..n_seed) holds the seeds, already
+// entered into the filter.
+template <int DT, int QR, int NS>
+__device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec<QR>& qv, int ef, Scratch& s, SearchState& st,
+                                                  Frontier<NS>& fr, int n_seed, int lane, bool* ambiguous) {
+  SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
+  const int cand_cap = s.cand_lds + s.cand_glob_cap;
+  const int S = row_stride(ix, 0);
+  int n = n_seed;
+  bool amb = false;
+  while (true) {
+    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    st.n_dist += n;
+    wave_sync();
+    for (int base = 0; base < n; base += 64) {
+      const int mine = base + lane;
+      const int at = mine < n ? mine : 0;
+      const float my_key = mine < n ? s.dbuf[at] : INFINITY;
+      const uint32_t my_id = s.nbuf[at];
+      unsigned long long todo = __ballot(mine < n && (st.n_acc < ef || st.lower > my_key));
+      while (todo != 0ull) {
+        const int j = __builtin_ctzll(todo);
+        todo &= todo - 1ull;
+        HeapEnt e;
+        e.key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+        e.id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+        if (st.n_acc < ef || st.lower > e.key) {
+          const bool twins = st.n_acc >= ef && frontier_max_twice<NS>(fr);
+          if (frontier_insert<NS>(fr, e.key, e.id, lane) != 2) {
+            amb = amb || twins;
+            if (st.cand_size >= cand_cap || st.n_acc >= s.log_cap) {
+              st.fail = 1;
+              return;
+            }
+            if (lane == 0) s.log[st.n_acc] = e;
+            st.n_acc = uni(st.n_acc + 1);
+            if (st.cand_size < s.cand_lds) {
+              LdsHeap cand_fast{s.cand};
+              coop_push<true>(cand_fast, st.cand_size, e, lane);
+            } else {
+              coop_push<true>(cand, st.cand_size, e, lane);
+            }
+            st.maxkey = uni(fmaxf(st.maxkey, e.key));
+            st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
+          }
+        }
+      }
+    }
+    st.top_size = st.n_acc < ef ? st.n_acc : ef;
+    int cid = -1;
+    if (st.cand_size > 0) {
+      wave_sync();
+      const HeapEnt c = uniform_ent(s.cand[0]);
+      if (!(c.key > st.lower)) {
+        cid = (int)c.id;
+        if (st.cand_size <= s.cand_lds) {
+          LdsHeap cand_fast{s.cand};
+          coop_pop<true>(cand_fast, st.cand_size, s.tree, lane);
+        } else {
+          coop_pop<true>(cand, st.cand_size, s.tree, lane);
+        }
+      }
+    }
+    wave_sync();
+    if (cid < 0) break;
+    st.n_hops += 1;
+    n = visit_lossy(link_row(ix, (uint32_t)cid, 0), S, s, lane);
+    wave_sync();
+  }
+  *ambiguous = amb;
+}
+
 // Greedy descent through levels from_level .. to_level+1 (hnswlib searchKnn upper
 // loop; cpp/include/cuda_search_kernels.cuh:22-66 in the reference): each sweep
 // scans the neighbour list captured at its start and moves to the strictly

@@ -61,6 +61,8 @@ struct SearchArgs {
   int fc_bits;  // log2 sets (two tags each) of the LDS visited filter of the sorted-set search, 0 = that search is off
   int fast_path;  // 0 = literal queues only (exact evaluation counters)
   int reverse;    // expand the farthest waiting candidate (reverse_cand); sorted-set pass only
+  int lean;       // literal pass: result set = sorted set with ids, visited = LDS filter of 2^lean sets
+                  // (no bitmap, evaluation counters include repeats); 0 = exact bitmap
 };
 
 struct BuildArgs {
@@ -95,10 +97,12 @@ __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t
 // search kernel the visited filter of the sorted-set search (fcache) takes the place of the
 // candidate queue and the literal search's visited cache.
 struct LdsPlan {
-  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, vcache, fcache, total;
+  size_t qlds, top, cand, sorted_id, sorted_key, out_id, out_key, nbuf, dbuf, vcache, fcache, lfilter, total;
 };
+// fc_bits: filter lying over the queue (build); lf_bits: filter of its own beside the queue (the
+// literal search on the sorted set)
 __host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds, int lcap, int n_sorted, int n_out,
-                                            int vc_bits = 0, int fc_bits = 0) {
+                                            int vc_bits = 0, int fc_bits = 0, int lf_bits = 0) {
   LdsPlan p;
   size_t o = 0;
   p.qlds = o;
@@ -115,6 +119,7 @@ __host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds
   p.out_key = o; o = align16(o + (size_t)n_out * 4);
   p.nbuf = o; o = align16(o + (size_t)lcap * 4);
   p.dbuf = o; o = align16(o + (size_t)lcap * 4);
+  p.lfilter = o; o = align16(o + (lf_bits > 0 ? ((size_t)4 << lf_bits) : 0));
   p.total = o;
   return p;
 }
@@ -240,10 +245,16 @@ template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
-  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.vc_bits);
+  const bool lean = NS > 0 && a.lean > 0;
+  const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, lean ? 0 : a.vc_bits, 0, a.lean);
   Scratch s;
-  s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
-  s.vc_bits = a.vc_bits;
+  if (lean) {
+    s.vcache = reinterpret_cast<uint16_t*>(smem + lp.lfilter);
+    s.vc_bits = a.lean;
+  } else {
+    s.vcache = a.vc_bits > 0 ? reinterpret_cast<uint16_t*>(smem + lp.vcache) : nullptr;
+    s.vc_bits = a.vc_bits;
+  }
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.top = reinterpret_cast<HeapEnt*>(smem + lp.top);
   s.cand = reinterpret_cast<HeapEnt*>(smem + lp.cand);
@@ -315,6 +326,42 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
     descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
 
+    int T;
+    bool literal = NS == 0;
+    bool have_result = false;  // s.nbuf / s.dbuf already hold the T answers in order
+    if (lean) {
+      Frontier<NS> fr;
+      frontier_init<NS>(fr, a.ef, lane);
+      filter_reset(s, lane);
+      visit_lossy_single(s, cur, lane);
+      if (lane == 0) s.nbuf[0] = cur;
+      wave_sync();
+      bool ambiguous = false;
+      search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous);
+      T = st.top_size < a.k ? st.top_size : a.k;
+      // The first T entries of the set are hnswlib's answer unless equal keys sit among them or
+      // across the cut, or the whole set is returned after an eviction had twins to choose
+      // from; then the result heap is replayed from the log, as below.
+      const bool replay = !st.fail && (frontier_tie_within<NS>(fr, a.ef, T, st.top_size, lane) ||
+                                       (ambiguous && T == st.top_size));
+      if (!st.fail && !replay) {
+        wave_sync();
+        frontier_dump<NS>(fr, a.ef, T, s.nbuf, s.dbuf, lane);
+        wave_sync();
+        have_result = true;
+      } else if (replay) {
+        __threadfence_block();
+        literal = true;
+        LdsHeap top{s.top};
+        int size = 0;
+        for (int i = 0; i < st.n_acc; ++i) {
+          const HeapEnt e = uniform_ent(s.log[i]);
+          coop_push<false>(top, size, e, lane);
+          if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
+        }
+        st.top_size = size;
+      }
+    } else {
     vcache_reset(s, lane);
     visit_single(s, st, cur, lane);
     if (lane == 0) s.nbuf[0] = cur;
@@ -324,8 +371,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     // the k best.  With the keys in registers: the entries of the log at or below the k-th
     // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the
     // literal heap decides: replay every accepted entry through it, pop down to k.
-    int T = st.top_size < a.k ? st.top_size : a.k;
-    bool literal = NS == 0;
+    T = st.top_size < a.k ? st.top_size : a.k;
     if (NS > 0 && !st.fail) {
       __threadfence_block();
       const float bound = topkeys_at<NS>(tk, T - 1, a.ef, reinterpret_cast<float*>(s.cand), lane);
@@ -342,22 +388,25 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
         st.top_size = size;
       }
     }
+    }
     if (literal) {
       LdsHeap top{s.top};
       while (st.top_size > a.k) coop_pop<false>(top, st.top_size, s.tree, lane);
       T = st.top_size;
     }
     wave_sync();
-    uint64_t* tie = nullptr;
-    if (ix.labels) {
-      // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
-      // whose first lcap entries hold the survivors themselves
-      tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
-      for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
+    if (!have_result) {
+      uint64_t* tie = nullptr;
+      if (ix.labels) {
+        // labels of the T survivors; with the keys in registers s.top aliases the queue's share,
+        // whose first lcap entries hold the survivors themselves
+        tie = reinterpret_cast<uint64_t*>(s.cand + (NS > 0 ? a.lcap : 0));
+        for (int e = lane; e < T; e += 64) tie[e] = ix.labels[s.top[e].id];
+        wave_sync();
+      }
+      rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
       wave_sync();
     }
-    rank_sort(s.top, tie, T, s.nbuf, s.dbuf, lane);
-    wave_sync();
     if (!a.hnswlib_dist && T > 0) {
       dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
       wave_sync();
@@ -383,7 +432,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
         a.stats[(size_t)qi * 4 + 3] = st.n_sweeps;
       }
     }
-    undo_visited(s, st, lane);
+    if (!lean) undo_visited(s, st, lane);
     wave_sync();
   }
 }

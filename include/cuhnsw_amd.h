@@ -121,6 +121,9 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   depending on how many queries the previous search handed over)
  *   "literal_spin_limit" polls one of its wavefronts may spend waiting for the first pass before
  *                   it leaves and the host answers the remaining queries afterwards (-1 = automatic)
+ *   "lean_literal"  visited set of the literal-queue pass: 0 = exact bitmap in HBM (one bit per point and
+ *                   wavefront), 2 = tag filter in LDS with the sorted set catching repeats, 1 = automatic
+ *                   (the bitmap while all bitmaps at work fit the L2 caches; default)
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)

@@ -42,8 +42,11 @@ def _check_parity(oracle, ix, e, q, k, ef, counters=True, dup_bound=3.0):
   LDS-only visited filter; queries that meet equal keys are repeated with literal queues)
   and the literal queues alone (fast_path = 0)."""
   o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
-  for fast in (2, 0):   # 2 = sorted-set pass whatever the batch size
+  # 2 = sorted-set pass whatever the batch size; 1 = default (a batch this small goes to the literal
+  # pass on the sorted set with ids and the LDS filter); 0 = literal queues with the exact bitmap
+  for fast in (2, 1, 0):
     e.set_tunable("fast_path", fast)
+    e.set_tunable("lean_literal", 2 if fast else 1)   # small test indexes would otherwise choose the bitmap
     g_ids, g_d, g_f = e.search_knn(q, k, ef)
     assert (g_f == o_f).all()
     for r in range(q.shape[0]):
@@ -65,6 +68,7 @@ def _check_parity(oracle, ix, e, q, k, ef, counters=True, dup_bound=3.0):
         assert (stats[:, 0] == o_cnt[:, 0]).all()
         assert e.last_search_repeats == 0
   e.set_tunable("fast_path", 1)
+  e.set_tunable("lean_literal", 1)
 
 
 CASES = [
