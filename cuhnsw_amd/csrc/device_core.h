@@ -8,14 +8,19 @@
 //     Replaces dot / squaresum / GetDistanceByVec of the reference
 //     (cpp/include/cuda_dist_kernels.cuh:13-124), which reduce over a 32-thread
 //     block through shared memory.
-//   * candidate queues live in LDS and reproduce libstdc++ heaps, each push / pop
-//     executed cooperatively by the wavefront (heap_coop.h);
-//     replaces the global-memory, thread-0 heap of the reference
-//     (cpp/include/cuda_heap_kernels.cuh:13-49) and its GetCand / CheckAlreadyExists
-//     scans (cpp/include/cuda_utils_kernels.cuh:50-151).
-//   * the visited set is an exact bitmap per resident wavefront (one bit per node,
-//     global memory, cleared through an undo list), not the lossy direct-mapped
-//     table of the reference (cpp/include/cuda_utils_kernels.cuh:185-210).
+//   * the search runs on ONE sorted set of (key, id, expanded) kept in registers
+//     (Frontier, search_level_fast): result set and candidate set of hnswlib at once, which
+//     is exact unless the layout of hnswlib's heaps would decide between equal keys; its
+//     visited filter is a two-way tag cache in LDS only (visit_lossy).  Replaces the
+//     global-memory, thread-0 heap of the reference (cpp/include/cuda_heap_kernels.cuh:13-49),
+//     its GetCand / CheckAlreadyExists scans (cpp/include/cuda_utils_kernels.cuh:50-151) and
+//     its lossy visited table (cpp/include/cuda_utils_kernels.cuh:185-210).
+//   * where equal keys do decide, the search is repeated with hnswlib's two priority queues
+//     reproduced move for move: candidate queue in LDS as a libstdc++ heap, each push / pop
+//     executed cooperatively by the wavefront (heap_coop.h), result set as sorted keys in
+//     registers plus a log (search_level), or as the sorted set with ids (search_level_lean);
+//     visited set either an exact bitmap per wavefront in global memory, cleared through an
+//     undo list, or the LDS filter.
 //
 // Canonical fp32 distance arithmetic: element i is accumulated with one fused
 // multiply-add into partial sum (i mod 64) in increasing i; the 64 partials are
