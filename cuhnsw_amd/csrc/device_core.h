@@ -196,22 +196,23 @@ __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const flo
 
 // one pass over 4*U rows starting at ids[r]: loads first, arithmetic after
 template <int DT, int R, int U, bool RAW>
-__device__ __forceinline__ void dist_pass(const float4* rows, int rowlen, const float4* q, const uint32_t* ids, int r, int n,
-                                          float* out, int g, int sub) {
-  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+__device__ __forceinline__ void dist_pass(const float4* rows, uint32_t rowlen, const float4* q, const uint32_t* ids, int r,
+                                          int n, float* out, int g, int sub) {
   float4 v[U][R];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int idx = r + 4 * u + g;
     const uint32_t id = ids[idx < n ? idx : n - 1];
-    const float4* p = rows + (size_t)id * rowlen;
+    const float4* p = rows + (uint64_t)id * rowlen;  // one 32x32->64 multiply-add
 #pragma unroll
     for (int k = 0; k < R; ++k) {
       // always one unconditional 16-byte load (a guarded one is split into four dword loads);
-      // chunks past the row end re-read chunk 0 and are zeroed afterwards
-      const int c = sub + 16 * k;
+      // a chunk past the row end re-reads chunk 0.  The query holds zeros there, which is all a
+      // dot product needs (finite data); for L2 the chunk is replaced by the query's own zeros.
+      // Rows are longer than 16 * (R / 2) chunks, so only the upper half of k can be past the end.
+      const uint32_t c = sub + 16 * k;
       const float4 t = p[c < rowlen ? c : 0];
-      v[u][k] = c < rowlen ? t : zero;
+      v[u][k] = (DT == DIST_DOT || k < R / 2 || c < rowlen) ? t : q[k];
     }
   }
 #pragma unroll
@@ -259,7 +260,7 @@ __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv
     for (int r = 0; r < n; r += 4) {
       const int idx = r + g;
       const uint32_t id = ids[idx < n ? idx : n - 1];
-      const float4* p = rows + (size_t)id * rowlen;
+      const float4* p = rows + (uint64_t)id * (uint32_t)rowlen;
       float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
       for (int k0 = 0; k0 < nk; k0 += B) {
         float4 v[B];
@@ -722,9 +723,10 @@ __device__ __forceinline__ bool frontier_max_twice(const Frontier<NS>& f) {
   const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f.k[N > 1 ? N - 2 : 0]), 63));
   return a == b;
 }
-// do two neighbouring keys coincide among sorted positions p, p+1 with p < upto and p+1 < count?
+// do two neighbouring keys coincide among sorted positions p, p+1 with from <= p < upto and p+1 < count?
 template <int NS>
-__device__ __forceinline__ bool frontier_tie_within(const Frontier<NS>& f, int ef, int upto, int count, int lane) {
+__device__ __forceinline__ bool frontier_tie_within(const Frontier<NS>& f, int ef, int upto, int count, int lane,
+                                                    int from = 0) {
   constexpr int N = NS > 0 ? NS : 1;
   const float next_first = __builtin_bit_cast(
       float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, f.k[0]), 0x130, 0xF, 0xF, false));  // wave_shl:1
@@ -733,7 +735,7 @@ __device__ __forceinline__ bool frontier_tie_within(const Frontier<NS>& f, int e
   for (int j = 0; j < N; ++j) {
     const int pos = lane * N + j - (64 * N - ef);
     const float nxt = j + 1 < N ? f.k[j + 1 < N ? j + 1 : 0] : next_first;
-    hit = hit || (pos >= 0 && pos < upto && pos + 1 < count && f.k[j] == nxt);
+    hit = hit || (pos >= from && pos < upto && pos + 1 < count && f.k[j] == nxt);
   }
   return __ballot(hit) != 0ull;
 }
@@ -814,8 +816,8 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 // entry evicted whose key equals the bound at the group's end.  (b) An eviction finds equal largest keys: which one leaves is the heap's
 // choice, and the one that leaves stays a live candidate of hnswlib as long as that key is
 // within the bound.  The search goes on, but gives up if it comes to expand an entry with such
-// a key, or ends while such a key is still within the bound.  (c) Equal keys among the k best
-// or across the cut: the caller's check.
+// a key, or ends while such a key is still within the bound.  (c) Equal keys across
+// the cut at k (the result heap's choice) or among the k best (listed by label): the caller's business.
 // far: expand the farthest waiting entry instead of the closest (the reference's
 // reverse_cand); that is no hnswlib search any more, equal keys simply keep their order of
 // arrival and nothing is ever given up.  BUILD likewise never gives up.
@@ -1052,6 +1054,31 @@ __device__ __forceinline__ void rank_sort(const HeapEnt* in, const uint64_t* tie
     out_id[rank] = me.id;
     out_key[rank] = me.key;
   }
+}
+
+// ids[0..n) with keys[0..n) ascending (LDS): puts the ids of every run of equal keys into the
+// order of their labels, which is how hnswlib's answer orders equal distances (its result queue
+// compares (distance, label) pairs).  tmp: n words of LDS.
+__device__ __forceinline__ void order_equal_keys(const DevIndex& ix, uint32_t* ids, const float* keys, int n, uint32_t* tmp,
+                                                 int lane) {
+  for (int e = lane; e < n; e += 64) tmp[e] = ids[e];
+  wave_sync();
+  for (int e = lane; e < n; e += 64) {
+    const float k = keys[e];
+    const uint32_t me = tmp[e];
+    const uint64_t ml = ix.labels ? ix.labels[me] : (uint64_t)me;
+    int rank = e;
+    for (int f = e - 1; f >= 0 && keys[f] == k; --f) {
+      const uint32_t o = tmp[f];
+      rank -= (ix.labels ? ix.labels[o] : (uint64_t)o) > ml ? 1 : 0;
+    }
+    for (int f = e + 1; f < n && keys[f] == k; ++f) {
+      const uint32_t o = tmp[f];
+      rank += (ix.labels ? ix.labels[o] : (uint64_t)o) < ml ? 1 : 0;
+    }
+    ids[rank] = me;
+  }
+  wave_sync();
 }
 
 // Collects from the log the entries that make up the k best: those with key <= bound.

@@ -391,8 +391,10 @@ class Engine {
       const bool side = concurrent_literal && max_slots_override <= 0;
       int side_slots = 0;
       // few queries need the literal pass (0.4 % of the 1.18M-point set's): one wavefront per CU
-      // serves them without taking room from the first pass; more when the last search needed more
-      const int per_cu = side_per_cu > 0 ? side_per_cu : (last_repeat_share < 0.02 ? 1 : (last_repeat_share < 0.06 ? 2 : 4));
+      // serves them without taking room from the first pass; two when the last search needed more
+      // (6.5 % on integer-valued 128-d data: 4.8 ms with one or two, 5.2 with four, 8.3 with eight —
+      // a literal wavefront's LDS is that of one and a half wavefronts of the first pass)
+      const int per_cu = side_per_cu > 0 ? side_per_cu : (last_repeat_share < 0.02 ? 1 : 2);
       if (side) {
         side_slots = std::min(num_cus * per_cu, a.nq);
         ensure_pool(std::max(side_slots, 1), glob_cap, 2 * glob_cap);

@@ -193,9 +193,12 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) s
     const int how =
         __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0));
     const int T0 = st.top_size < a.k ? st.top_size : a.k;
-    // equal keys among the k best or across the cut: order and membership follow the
-    // (distance, label) rule and the result heap, which the literal search reproduces
-    const bool gave_up = how == 1 || (how == 2 && !a.reverse && frontier_tie_within<NS>(fr, a.ef, T0, st.top_size, lane));
+    // Equal keys across the cut at k: which of them stays is up to the result heap, which the
+    // literal search reproduces.  Equal keys among the k best: the answer lists them by label.
+    const bool cut_tie = how == 2 && !a.reverse && frontier_tie_within<NS>(fr, a.ef, T0, st.top_size, lane, T0 - 1);
+    const int inner_tie = __builtin_amdgcn_readfirstlane(
+        (how == 2 && !a.reverse && frontier_tie_within<NS>(fr, a.ef, T0 - 1, st.top_size, lane)) ? 1 : 0);
+    const bool gave_up = how == 1 || cut_tie || (inner_tie && T0 > (1 << a.fc_bits));  // (the filter's LDS is the sort's buffer)
     if (gave_up) {
       if (lane == 0) {
         const int slot = atomicAdd(a.repeats, 1);
@@ -206,6 +209,7 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) s
       wave_sync();
       frontier_dump<NS>(fr, a.ef, T, s.nbuf, s.dbuf, lane);
       wave_sync();
+      if (inner_tie) order_equal_keys(ix, s.nbuf, s.dbuf, T, reinterpret_cast<uint32_t*>(s.vcache), lane);
       if (!a.hnswlib_dist && T > 0) {
         dist_list<DT, QR, true>(ix, qv, s.qlds, s.nbuf, T, s.dbuf, lane);
         wave_sync();
@@ -339,15 +343,17 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
       bool ambiguous = false;
       search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous);
       T = st.top_size < a.k ? st.top_size : a.k;
-      // The first T entries of the set are hnswlib's answer unless equal keys sit among them or
-      // across the cut, or the whole set is returned after an eviction had twins to choose
-      // from; then the result heap is replayed from the log, as below.
-      const bool replay = !st.fail && (frontier_tie_within<NS>(fr, a.ef, T, st.top_size, lane) ||
-                                       (ambiguous && T == st.top_size));
+      // The first T entries of the set (equal keys among them in label order) are hnswlib's
+      // answer unless equal keys sit across the cut, or the whole set is returned after an
+      // eviction had twins to choose from; then the result heap is replayed from the log, as below.
+      const bool inner_tie = !st.fail && frontier_tie_within<NS>(fr, a.ef, T - 1, st.top_size, lane);
+      const bool replay = !st.fail && (frontier_tie_within<NS>(fr, a.ef, T, st.top_size, lane, T - 1) ||
+                                       (ambiguous && T == st.top_size) || (inner_tie && T > (1 << a.lean)));
       if (!st.fail && !replay) {
         wave_sync();
         frontier_dump<NS>(fr, a.ef, T, s.nbuf, s.dbuf, lane);
         wave_sync();
+        if (inner_tie) order_equal_keys(ix, s.nbuf, s.dbuf, T, reinterpret_cast<uint32_t*>(s.vcache), lane);
         have_result = true;
       } else if (replay) {
         __threadfence_block();

@@ -117,7 +117,7 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
  *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
  *                   (default), 0 = after it
- *   "literal_per_cu" wavefronts per CU of that concurrent literal pass (0 = automatic: 1, 2 or 4
+ *   "literal_per_cu" wavefronts per CU of that concurrent literal pass (0 = automatic: 1 or 2
  *                   depending on how many queries the previous search handed over)
  *   "literal_spin_limit" polls one of its wavefronts may spend waiting for the first pass before
  *                   it leaves and the host answers the remaining queries afterwards (-1 = automatic)

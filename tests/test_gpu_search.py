@@ -291,21 +291,29 @@ def test_followed_up_ties_match_the_oracle_on_quantised_data(oracle, tmp_path, s
   q = integer_vectors(700, d, seed=seed + 50, hi=hi)
   mult = 1 / np.log(8)
   levels = _levels(n, mult, seed + 7)
-  ix = oracle.OracleIndex("l2").build(x, levels, 8, 16, 50, mult)
-  p = str(tmp_path / "qd.idx")
-  ix.save(p)
-  e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
-  e.load_index(p)
-  e.set_tunable("fast_path", 2)
-  answered_by_first_pass = 0
-  for k, ef in ((10, 64), (10, 300), (1, 16), (100, 100), (32, 33), (5, 319), (10, 700)):
-    o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
-    g_ids, g_d, g_f, stats = _device_search(e, q, k, ef)
-    assert (g_f == o_f).all()
-    for r in range(q.shape[0]):
-      f = o_f[r]
-      assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d k %d ef %d" % (r, k, ef)
-      assert (g_d[r, :f] == o_d[r, :f]).all()
-    assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
-    answered_by_first_pass += q.shape[0] - e.last_search_repeats
-  assert answered_by_first_pass > 0
+  base = oracle.OracleIndex("l2").build(x, levels, 8, 16, 50, mult)
+  # the same graph under labels that reverse the order of the ids: equal distances among the
+  # k best are listed by label, so the two answers differ in exactly those places
+  labels = (np.uint64(3) * (n - 1 - np.arange(n, dtype=np.uint64)) + np.uint64(7))
+  up = np.concatenate([np.concatenate([[len(base.links(i, l))], np.pad(base.links(i, l), (0, 8 - len(base.links(i, l))))])
+                       for i in range(n) for l in range(1, levels[i] + 1)]).astype(np.uint32)
+  relabelled = oracle.OracleIndex("l2").from_arrays(x, levels, base.links0(), up, 8, 16, base.maxlevel, base.enterpoint,
+                                                    labels=labels)
+  for tag, ix in (("ids", base), ("labels", relabelled)):
+    p = str(tmp_path / ("qd_%s.idx" % tag))
+    ix.save(p)
+    e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
+    e.load_index(p)
+    e.set_tunable("fast_path", 2)
+    answered_by_first_pass = 0
+    for k, ef in ((10, 64), (10, 300), (1, 16), (100, 100), (32, 33), (5, 319), (10, 700)):
+      o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
+      g_ids, g_d, g_f, stats = _device_search(e, q, k, ef)
+      assert (g_f == o_f).all()
+      for r in range(q.shape[0]):
+        f = o_f[r]
+        assert (g_ids[r, :f] == o_ids[r, :f]).all(), "%s query %d k %d ef %d" % (tag, r, k, ef)
+        assert (g_d[r, :f] == o_d[r, :f]).all()
+      assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
+      answered_by_first_pass += q.shape[0] - e.last_search_repeats
+    assert answered_by_first_pass > 0
