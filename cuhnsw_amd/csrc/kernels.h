@@ -154,10 +154,11 @@ __host__ __device__ inline FastLdsPlan plan_fast_lds(int qr, int Dp, int lcap, i
 // First pass of a search batch: every query on the sorted set in registers (ef < 64*NS).
 // A query in which two equal keys meet is not answered here: its index is appended to
 // a.redo (a.repeats counts them) and the literal search_kernel answers it afterwards.
-// (with five keys per lane and the query in at most two registers the kernel is held to 80
-// registers, six wavefronts per SIMD; the other shapes would spill)
+// (with at most five keys per lane and the query in at most two float4 registers the kernel is
+// held to 72 registers, seven wavefronts per SIMD, at the price of up to five spilled registers;
+// eight wavefronts are no faster, the other shapes would spill heavily)
 template <int DT, int QR, int NS>
-__global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 6 : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
+__global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 7 : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
   const FastLdsPlan lp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
@@ -318,6 +319,9 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     }
     qi = __builtin_amdgcn_readfirstlane(qi);
     if (qi < 0) break;
+    // beside the first pass a literal wavefront is one among a few dozen on its CU and its query
+    // is on the batch's critical path: it goes first whenever it has an instruction ready
+    if (a.live) __builtin_amdgcn_s_setprio(3);
     QVec<QR> qv;
     load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
     SearchState st;
@@ -440,6 +444,7 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
     }
     if (!lean) undo_visited(s, st, lane);
     wave_sync();
+    if (a.live) __builtin_amdgcn_s_setprio(0);  // waiting for the next query is nobody's critical path
   }
 }
 

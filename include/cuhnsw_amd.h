@@ -45,7 +45,8 @@ int cuhnsw_init(cuhnsw_engine* e, const char* opt_path);
 /* void CuHNSW::SetData(const float* data, int num_data, int num_dims)
  * (cpp/src/cuhnsw_base.cu:108-128).  data: row-major float32 [num_data x
  * num_dims] in host memory.  The engine keeps its own copy (the reference keeps
- * the caller's raw pointer). */
+ * the caller's raw pointer).  Values are expected to be finite: what a search
+ * returns for rows that hold infinities or NaNs is not specified. */
 int cuhnsw_set_data(cuhnsw_engine* e, const float* data, int num_data, int num_dims);
 
 /* void CuHNSW::SetRandomLevels(const int* levels) (cpp/src/cuhnsw_base.cu:130-156):
