@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--storage fp32|fp16] [--no-cpu]
 
 Workload (default C2): the GloVe-50-shaped angular configuration — 1 183 514 x 50
 float32 vectors from the seeded 1000-centre Gaussian mixture, L2-normalised,
@@ -39,6 +39,9 @@ def main():
   ap.add_argument("--nq", type=int, default=None)
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
   ap.add_argument("--ef", type=int, default=None, help="ef_search (default: the configuration's headline value)")
+  ap.add_argument("--storage", choices=["fp32", "fp16"], default="fp32",
+                  help="element type of the vectors in device memory; fp16 = an index over the vectors rounded "
+                       "to fp16, arithmetic stays fp32 (the default is the configuration the metric is quoted on)")
   ap.add_argument("--copy-calibration", action="store_true",
                   help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   args = ap.parse_args()
@@ -74,6 +77,8 @@ def main():
     json.dump(opt, f)
   eng = capi.Engine()
   assert eng.init(opt_path) == 0
+  if args.storage == "fp16":
+    eng.set_tunable("fp16_storage", 1)
   t0 = time.time()
   eng.set_data(data)
   upload_s = time.time() - t0
@@ -166,14 +171,14 @@ def main():
     del ql, l_nns, l_dist, l_found
 
   avg_kernel_ms = float(np.mean(kernel_ms))
-  gather_bytes = int(st[:, 0].sum()) * 4 * d
+  gather_bytes = int(st[:, 0].sum()) * (2 if args.storage == "fp16" else 4) * d
   # HBM bytes of one search of the default batch, measured once with two rocprofv3 --pmc runs of
   # this very command (FETCH_SIZE 2 304 000 + 8 044 KiB over both search kernels, scaled by 2.0:
   # a 256 MiB device copy reads 131 084 on that counter; WRITE_SIZE 4 127 + 218 KiB, scaled by
   # 1.0: the copy writes 262 144).  It cannot be measured from inside this process; other
   # workloads report null.
   traffic = None
-  if args.workload == "C2" and args.n is None and args.nq is None and ef == 300:
+  if args.workload == "C2" and args.n is None and args.nq is None and ef == 300 and args.storage == "fp32":
     traffic = int((2304000 + 8044) * 1024 * 2.0 + (4127 + 218) * 1024 * 1.0)
   achieved = gather_bytes / (avg_kernel_ms * 1e-3) / 1e9
   out = {
@@ -186,7 +191,9 @@ def main():
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
       "dtype": "f32", "data": "synthetic",
       "config": {"workload": "%s: %dx%d %s max_m=%d max_m0=%d ef_construction=%d; %d queries topk=%d ef_search=%d" % (
-          args.workload, n, d, o["dist_type"], o["max_m"], o["max_m0"], o["ef_construction"], nq, k, ef)},
+          args.workload, n, d, o["dist_type"], o["max_m"], o["max_m0"], o["ef_construction"], nq, k, ef) + (
+              "; vectors stored as fp16 (recall is against the exact neighbours of the unrounded vectors)"
+              if args.storage == "fp16" else "")},
       "build_seconds": build_s,
       "recall_at_k": recall,
       "upload_seconds": upload_s, "datagen_seconds": gen_s,

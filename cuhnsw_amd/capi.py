@@ -128,7 +128,10 @@ class Engine:
     return ms.value
 
   def set_tunable(self, name, value):
-    if self._l.cuhnsw_set_tunable(self._h, name.encode(), float(value)) != 0:
+    rc = self._l.cuhnsw_set_tunable(self._h, name.encode(), float(value))
+    if rc == -2:
+      raise RuntimeError("tunable " + name + " has to be set before set_data / load_index")
+    if rc != 0:
       raise RuntimeError("unknown tunable " + name)
 
   num_data = property(lambda s: s._l.cuhnsw_num_data(s._h))

@@ -70,7 +70,9 @@ class CuHNSWBind {
   int EnterPoint() const { return cuhnsw_enter_point(obj_); }
   double LastBuildSeconds() const { return cuhnsw_last_build_seconds(obj_); }
   void SetTunable(std::string name, double value) {
-    if (cuhnsw_set_tunable(obj_, name.c_str(), value) != 0) throw std::runtime_error("unknown tunable " + name);
+    const int rc = cuhnsw_set_tunable(obj_, name.c_str(), value);
+    if (rc == -2) throw std::runtime_error("tunable " + name + " has to be set before set_data / load_index");
+    if (rc != 0) throw std::runtime_error("unknown tunable " + name);
   }
 
  private:

@@ -37,7 +37,7 @@
 namespace cuhnsw_amd {
 
 struct DevIndex {
-  const float* vectors;      // N x Dp, rows zero padded to Dp (multiple of 32 floats)
+  const void* vectors;       // N x Dp, rows zero padded to Dp (multiple of 32 elements); fp32, or fp16 when half != 0
   const uint64_t* labels;    // N, or null when labels are the internal ids
   uint32_t* links0;          // N x S0
   uint32_t* linksU;          // upper rows x SU
@@ -47,6 +47,7 @@ struct DevIndex {
   float* distsU;             // build only
   int N, D, Dp, S0, SU, max_m, max_m0, maxlevel;
   uint32_t enterpoint;
+  int half;                  // vectors are stored as fp16 (all arithmetic stays fp32 on the stored values)
 };
 
 // per resident wavefront scratch: LDS pointers + this wavefront's global slot
@@ -148,6 +149,19 @@ __device__ __forceinline__ void acc4(const float4 q, const float4 v, float& ax, 
     aw = __builtin_fmaf(tw, tw, aw);
   }
 }
+// One chunk (four consecutive elements) of stored vectors: 16 bytes of fp32, or 8 bytes of fp16
+// widened to fp32 (exact).  `chunk` counts chunks from the start of the array.
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load_chunk_f32(const void* base, uint64_t chunk) {
+  return reinterpret_cast<const float4*>(base)[chunk];
+}
+__device__ __forceinline__ float4 load_chunk_f16(const void* base, uint64_t chunk) {
+  const half4_t h = reinterpret_cast<const half4_t*>(base)[chunk];
+  const floatx4_t f = __builtin_convertvector(h, floatx4_t);
+  return make_float4(f.x, f.y, f.z, f.w);
+}
+
 // RAW = false: ordering key (1 - dot | squared L2); RAW = true: API value (-dot | squared L2)
 template <int DT, bool RAW>
 __device__ __forceinline__ float finish16(float ax, float ay, float az, float aw) {
@@ -195,23 +209,24 @@ __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const flo
 }
 
 // one pass over 4*U rows starting at ids[r]: loads first, arithmetic after
-template <int DT, int R, int U, bool RAW>
-__device__ __forceinline__ void dist_pass(const float4* rows, uint32_t rowlen, const float4* q, const uint32_t* ids, int r,
+template <int DT, int R, int U, bool RAW, bool HALF>
+__device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, const float4* q, const uint32_t* ids, int r,
                                           int n, float* out, int g, int sub) {
   float4 v[U][R];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int idx = r + 4 * u + g;
     const uint32_t id = ids[idx < n ? idx : n - 1];
-    const float4* p = rows + (uint64_t)id * rowlen;  // one 32x32->64 multiply-add
+    const uint64_t first = (uint64_t)id * rowlen;  // one 32x32->64 multiply-add
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-      // always one unconditional 16-byte load (a guarded one is split into four dword loads);
-      // a chunk past the row end re-reads chunk 0.  The query holds zeros there, which is all a
-      // dot product needs (finite data); for L2 the chunk is replaced by the query's own zeros.
-      // Rows are longer than 16 * (R / 2) chunks, so only the upper half of k can be past the end.
+      // always one unconditional load (a guarded one is split into dword loads); a chunk past
+      // the row end re-reads chunk 0.  The query holds zeros there, which is all a dot product
+      // needs (finite data); for L2 the chunk is replaced by the query's own zeros.  Rows are
+      // longer than 16 * (R / 2) chunks, so only the upper half of k can be past the end.
       const uint32_t c = sub + 16 * k;
-      const float4 t = p[c < rowlen ? c : 0];
+      const uint64_t at = first + (c < rowlen ? c : 0);
+      const float4 t = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
       v[u][k] = (DT == DIST_DOT || k < R / 2 || c < rowlen) ? t : q[k];
     }
   }
@@ -226,13 +241,49 @@ __device__ __forceinline__ void dist_pass(const float4* rows, uint32_t rowlen, c
   }
 }
 
+// long rows: 16 lanes still own one row (the summation order is tied to 16 lanes), so a lane
+// has rowlen/16 chunks to fetch; they are issued eight at a time to keep eight loads per lane
+// in flight, the query chunks come from LDS
+template <int DT, bool RAW, bool HALF>
+__device__ __forceinline__ void dist_long(const void* rows, int rowlen, const float4* qlds, const uint32_t* ids, int n,
+                                          float* out, int g, int sub) {
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int nk = (rowlen + 15) >> 4;
+  constexpr int B = 8;
+  for (int r = 0; r < n; r += 4) {
+    const int idx = r + g;
+    const uint32_t id = ids[idx < n ? idx : n - 1];
+    const uint64_t first = (uint64_t)id * (uint32_t)rowlen;
+    float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
+    for (int k0 = 0; k0 < nk; k0 += B) {
+      float4 v[B];
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int c = sub + 16 * (k0 + b);
+        const uint64_t at = first + (c < rowlen ? c : 0);  // unconditional load
+        const float4 t = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
+        v[b] = c < rowlen ? t : zero;
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        // chunks past the row end multiply zeros (the LDS copy is padded to a multiple of 16
+        // chunks, so only indices below that are read)
+        const float4 qq = (k0 + b < nk) ? qlds[sub + 16 * (k0 + b)] : zero;
+        acc4<DT>(qq, v[b], ax, ay, az, aw);
+      }
+    }
+    const float key = finish16<DT, RAW>(ax, ay, az, aw);
+    if (sub == 0 && idx < n) out[idx] = key;
+  }
+}
+
 // keys of ids[0..n) (LDS) against the query -> out[0..n) (LDS).  n is wavefront-uniform.
-template <int DT, int QR, bool RAW>
-__device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds,
-                                          const uint32_t* ids, int n, float* out, int lane) {
+template <int DT, int QR, bool RAW, bool HALF>
+__device__ __forceinline__ void dist_list_t(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds, const uint32_t* ids,
+                                            int n, float* out, int lane) {
   const int g = lane >> 4, sub = lane & 15;
   const int rowlen = ix.Dp >> 2;
-  const float4* rows = reinterpret_cast<const float4*>(ix.vectors);
+  const void* rows = ix.vectors;
   if (QR > 0) {
     constexpr int R = QR > 0 ? QR : 1;
     constexpr int UMAX = R == 1 ? 4 : (R == 2 ? 2 : 1);  // groups of 4 rows in flight
@@ -240,48 +291,26 @@ __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv
     while (r < n) {
       const int rem = n - r;
       if (UMAX >= 4 && rem > 8) {
-        dist_pass<DT, R, (UMAX >= 4 ? 4 : 1), RAW>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        dist_pass<DT, R, (UMAX >= 4 ? 4 : 1), RAW, HALF>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
         r += 16;
       } else if (UMAX >= 2 && rem > 4) {
-        dist_pass<DT, R, (UMAX >= 2 ? 2 : 1), RAW>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        dist_pass<DT, R, (UMAX >= 2 ? 2 : 1), RAW, HALF>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
         r += 8;
       } else {
-        dist_pass<DT, R, 1, RAW>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        dist_pass<DT, R, 1, RAW, HALF>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
         r += 4;
       }
     }
   } else {
-    // long rows: 16 lanes still own one row (the summation order is tied to 16 lanes), so
-    // a lane has rowlen/16 chunks to fetch; they are issued eight at a time to keep eight
-    // 16-byte loads per lane in flight, the query chunks come from LDS
-    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int nk = (rowlen + 15) >> 4;
-    constexpr int B = 8;
-    for (int r = 0; r < n; r += 4) {
-      const int idx = r + g;
-      const uint32_t id = ids[idx < n ? idx : n - 1];
-      const float4* p = rows + (uint64_t)id * (uint32_t)rowlen;
-      float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
-      for (int k0 = 0; k0 < nk; k0 += B) {
-        float4 v[B];
-#pragma unroll
-        for (int b = 0; b < B; ++b) {
-          const int c = sub + 16 * (k0 + b);
-          const float4 t = p[c < rowlen ? c : 0];  // unconditional 16-byte load
-          v[b] = c < rowlen ? t : zero;
-        }
-#pragma unroll
-        for (int b = 0; b < B; ++b) {
-          // chunks past the row end multiply zeros (the LDS copy is padded to a multiple of 16
-          // chunks, so only indices below that are read)
-          const float4 qq = (k0 + b < nk) ? qlds[sub + 16 * (k0 + b)] : zero;
-          acc4<DT>(qq, v[b], ax, ay, az, aw);
-        }
-      }
-      const float key = finish16<DT, RAW>(ax, ay, az, aw);
-      if (sub == 0 && idx < n) out[idx] = key;
-    }
+    dist_long<DT, RAW, HALF>(rows, rowlen, qlds, ids, n, out, g, sub);
   }
+}
+// (the element type of the stored vectors is a property of the index: one scalar branch per list)
+template <int DT, int QR, bool RAW>
+__device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds,
+                                          const uint32_t* ids, int n, float* out, int lane) {
+  if (uni(ix.half) != 0) dist_list_t<DT, QR, RAW, true>(ix, qv, qlds, ids, n, out, lane);
+  else dist_list_t<DT, QR, RAW, false>(ix, qv, qlds, ids, n, out, lane);
 }
 
 __device__ __forceinline__ const uint32_t* link_row(const DevIndex& ix, uint32_t node, int level) {

@@ -88,6 +88,7 @@ class Engine {
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
+  bool storage_half = false;  // vectors live in HBM as fp16 (set before set_data / load_index)
   int fast_path = 1;     // 0: search with the literal queues only; 1: sorted-set pass first when the batch is
                          // larger than one round of literal wavefronts; 2: always
   int last_repeats = 0;  // queries of the last search that were repeated with the literal queues
@@ -161,6 +162,7 @@ class Engine {
     ix.levels = d_levels.p;
     ix.dists0 = dists0;
     ix.distsU = distsU;
+    ix.half = storage_half ? 1 : 0;
     ix.N = host.N; ix.D = host.D; ix.Dp = Dp; ix.S0 = host.S0; ix.SU = host.SU;
     ix.max_m = host.max_m; ix.max_m0 = host.max_m0; ix.maxlevel = host.maxlevel;
     ix.enterpoint = host.enterpoint;
@@ -181,9 +183,25 @@ class Engine {
 
   // vectors go up as one contiguous copy (a pitched copy from pageable memory crawls row by
   // row); rows that need padding are spread out by a small kernel on the device
+  // With fp16 storage the host copy is rounded to the stored values first: everything downstream
+  // (the saved file, a CPU search of that file) then sees exactly the vectors the kernels see.
   void upload_vectors() {
     Dp = padded_dims(host.D);
     const size_t n = (size_t)host.N;
+    if (storage_half) {
+      for (float& x : host.vectors) x = (float)(_Float16)x;
+      d_vectors.reserve((n * Dp + 1) / 2);
+      DevBuf<float> raw;
+      raw.reserve(n * host.D);
+      HIP_CHECK(hipMemcpyAsync(raw.p, host.vectors.data(), n * host.D * sizeof(float), hipMemcpyHostToDevice, stream));
+      HIP_CHECK(hipMemsetAsync(d_vectors.p, 0, n * Dp * sizeof(_Float16), stream));
+      const long long work = (long long)n * host.D;
+      hipLaunchKernelGGL(pad_rows_half_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, raw.p,
+                         reinterpret_cast<_Float16*>(d_vectors.p), (long long)n, host.D, Dp);
+      HIP_CHECK(hipGetLastError());
+      HIP_CHECK(hipStreamSynchronize(stream));
+      return;
+    }
     d_vectors.reserve(n * Dp);
     if (Dp == host.D) {
       HIP_CHECK(hipMemcpyAsync(d_vectors.p, host.vectors.data(), n * Dp * sizeof(float), hipMemcpyHostToDevice, stream));
@@ -805,6 +823,10 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "literal_spin_limit") e->impl.spin_limit_override = (int)value;
   else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(0, std::min(8, (int)value));
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
+  else if (n == "fp16_storage") {
+    if (e->impl.have_data && e->impl.storage_half != (value != 0.0)) return -2;  // only before the vectors are there
+    e->impl.storage_half = value != 0.0;
+  }
   else return -1;
   return 0;
 }

@@ -449,25 +449,35 @@ __global__ void __launch_bounds__(64) search_kernel(DevIndex ix, SearchArgs a) {
 }
 
 // loads the (zero padded, 128-byte aligned) vector of a stored node as the "query"
-template <int QR>
-__device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, const DevIndex& ix, uint32_t node, int lane) {
+template <int QR, bool HALF>
+__device__ __forceinline__ void load_node_query_t(QVec<QR>& qv, float4* qlds, const DevIndex& ix, uint32_t node, int lane) {
   const int rowlen = ix.Dp >> 2;
-  const float4* p = reinterpret_cast<const float4*>(ix.vectors) + (size_t)node * rowlen;
+  const uint64_t first = (uint64_t)node * (uint32_t)rowlen;
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   if (QR > 0) {
     const int sub = lane & 15;
 #pragma unroll
     for (int k = 0; k < (QR > 0 ? QR : 1); ++k) {
       const int c = sub + 16 * k;
-      const float4 t = p[c < rowlen ? c : 0];  // unconditional 16-byte load
+      const uint64_t at = first + (c < rowlen ? c : 0);  // unconditional load
+      const float4 t = HALF ? load_chunk_f16(ix.vectors, at) : load_chunk_f32(ix.vectors, at);
       qv.q[k] = c < rowlen ? t : zero;
     }
   } else {
     const int chunks = (rowlen + 15) / 16 * 16;
     wave_sync();
-    for (int c = lane; c < chunks; c += 64) qlds[c] = c < rowlen ? p[c] : zero;
+    for (int c = lane; c < chunks; c += 64) {
+      const uint64_t at = first + (c < rowlen ? c : 0);
+      const float4 t = HALF ? load_chunk_f16(ix.vectors, at) : load_chunk_f32(ix.vectors, at);
+      qlds[c] = c < rowlen ? t : zero;
+    }
     wave_sync();
   }
+}
+template <int QR>
+__device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, const DevIndex& ix, uint32_t node, int lane) {
+  if (uni(ix.half) != 0) load_node_query_t<QR, true>(qv, qlds, ix, node, lane);
+  else load_node_query_t<QR, false>(qv, qlds, ix, node, lane);
 }
 
 // Neighbour selection (HNSW Alg. 4 / hnswlib getNeighborsByHeuristic2) with the two
@@ -786,6 +796,15 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
     if (lane == 0) *cnt = 0;
     wave_sync();
   }
+}
+
+// Upload helper for fp16 storage: N x D floats into rows of Dp halves (the padding was zeroed before).
+__global__ void __launch_bounds__(256) pad_rows_half_kernel(const float* src, _Float16* dst, long long n, int D, int Dp) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * D) return;
+  const long long row = i / D;
+  const int col = (int)(i - row * D);
+  dst[row * Dp + col] = (_Float16)src[i];  // round to nearest even; the host rounds its copy the same way
 }
 
 // Upload helper: copies N x D floats into rows of Dp floats (the padding was zeroed before).

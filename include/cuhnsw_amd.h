@@ -128,7 +128,13 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)
- * returns non-zero for an unknown name */
+ *   "fp16_storage"  1 = the vectors are kept in device memory as fp16 (the reference's switched-off
+ *                   HALF_PRECISION idea, cpp/include/types.hpp:9-28).  The index then IS an index over
+ *                   the vectors rounded to fp16 (nearest even; magnitudes beyond 65504 become
+ *                   infinite): queries and all arithmetic stay fp32, save_index writes the rounded
+ *                   vectors, and a CPU search of that file returns the same ids and distances.
+ *                   Has to be set before set_data / load_index (returns -2 afterwards).  Default 0.
+ * returns -1 for an unknown name */
 int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value);
 
 #ifdef __cplusplus
