@@ -173,13 +173,13 @@ def main():
   avg_kernel_ms = float(np.mean(kernel_ms))
   gather_bytes = int(st[:, 0].sum()) * (2 if args.storage == "fp16" else 4) * d
   # HBM bytes of one search of the default batch, measured once with two rocprofv3 --pmc runs of
-  # this very command (FETCH_SIZE 2 304 000 + 8 044 KiB over both search kernels, scaled by 2.0:
-  # a 256 MiB device copy reads 131 084 on that counter; WRITE_SIZE 4 127 + 218 KiB, scaled by
+  # this very command (FETCH_SIZE 2 009 400 + 7 308 KiB over both search kernels, scaled by 2.0:
+  # a 256 MiB device copy reads 131 084 on that counter; WRITE_SIZE 7 584 + 196 KiB, scaled by
   # 1.0: the copy writes 262 144).  It cannot be measured from inside this process; other
   # workloads report null.
   traffic = None
   if args.workload == "C2" and args.n is None and args.nq is None and ef == 300 and args.storage == "fp32":
-    traffic = int((2304000 + 8044) * 1024 * 2.0 + (4127 + 218) * 1024 * 1.0)
+    traffic = int((2009400 + 7308) * 1024 * 2.0 + (7584 + 196) * 1024 * 1.0)
   achieved = gather_bytes / (avg_kernel_ms * 1e-3) / 1e9
   out = {
       "metric": "batch search QPS at recall@%d (%s: %dx%d %s), with build seconds" % (

@@ -330,16 +330,19 @@ class Engine {
     return bits;
   }
 
-  // log2 sets (two 16-bit tags each) of the LDS visited filter of the sorted-set search.  A
-  // search evaluates about ef * max_m0 / 5 nodes; the filter gets room for somewhat more than
-  // that (4 KB at ef = 300, max_m0 = 24), and twice as much when a repeated evaluation is
-  // expensive (rows of 2 KB and more).  0 when ids do not fit the tags.
+  // log2 of the size in 32-bit words (two 16-bit tags each; a set is two words, four ways) of
+  // the LDS visited filter of the sorted-set search.  A search at ef = 300 evaluates 1 100 to
+  // 1 300 distinct nodes on the million-point sets (max_m0 24 and 32 alike), about 800 at
+  // ef = 100; the filter gets 4 * ef + 512 entries rounded up to a power of two (1 024 up to
+  // ef = 128, 2 048 = 4 KB up to ef = 384), and twice as much when a repeated evaluation is
+  // expensive (rows of 2 KB and more).  More costs occupancy and is slower, less repeats more.
+  // 0 when ids do not fit the tags.
   int auto_fc_bits(int ef) const {
-    long long want = filter_entries > 0 ? filter_entries : (long long)ef * host.max_m0 / 4;
+    long long want = filter_entries > 0 ? filter_entries : 4ll * ef + 512;
     if (filter_entries <= 0 && Dp >= 512) want *= 2;
     int bits = 8;
     while ((2ll << bits) < want && bits < 13) ++bits;
-    if (((unsigned)host.N >> bits) >= 0xFFFFu) return 0;
+    if (((unsigned)host.N >> (bits - 1)) >= 0xFFFFu) return 0;  // tags are 16 bits wide, sets 64
     return bits;
   }
 
@@ -388,7 +391,7 @@ class Engine {
       const size_t room = per_cu > 0 ? (size_t)(150 * 1024) / per_cu : 0;
       const size_t other = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, 0, 0, 0).total + 256;
       while (a.lean < 13 && other + ((size_t)4 << (a.lean + 1)) <= std::min<size_t>(room, 60 * 1024) &&
-             (((unsigned)host.N >> (a.lean + 1)) < 0xFFFFu))
+             (((unsigned)host.N >> a.lean) < 0xFFFFu))
         ++a.lean;
     }
     const LdsPlan lp = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, a.cand_lds, a.lcap, 0, 0, a.lean ? 0 : a.vc_bits, 0, a.lean);
