@@ -406,8 +406,17 @@ class Engine {
     if (NS > 0 && a.fast_path && a.fc_bits > 0 && (a.fast_path > 1 || a.nq > lit_slots)) {  // (reverse_cand: fast_path is 2)
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
-      const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
       auto fast_kernel = search_fast_kernel<DT, QR, NS>;
+      // the filter must not be what limits the wavefronts per CU: half the filter repeats more
+      // evaluations but is the faster choice wherever it buys occupancy (10 M x 96, ef = 512,
+      // five wavefronts per SIMD by registers: 46.8 ms with 8 KB of filter, 45.2 ms with 4 KB)
+      while (filter_entries <= 0 && a.fc_bits > 9) {
+        const int now = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits).total);
+        const int with_half = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits - 1).total);
+        if (with_half * 20 < now * 23) break;  // less than 15 % more
+        --a.fc_bits;
+      }
+      const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
       int slots = resident_slots(fast_kernel, fp.total);
       const bool side = concurrent_literal && max_slots_override <= 0;
       int side_slots = 0;

@@ -156,9 +156,10 @@ __host__ __device__ inline FastLdsPlan plan_fast_lds(int qr, int Dp, int lcap, i
 // a.redo (a.repeats counts them) and the literal search_kernel answers it afterwards.
 // (with at most five keys per lane and the query in at most two float4 registers the kernel is
 // held to 72 registers, seven wavefronts per SIMD, at the price of up to five spilled registers;
-// eight wavefronts are no faster, the other shapes would spill heavily)
+// eight wavefronts are no faster; with eight keys per lane it fits 96 registers, five wavefronts
+// per SIMD, without spilling; the other shapes would spill heavily)
 template <int DT, int QR, int NS>
-__global__ void __launch_bounds__(64, (NS <= 5 && QR >= 1 && QR <= 2) ? 7 : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
+__global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS == 8 ? 5 : 1)) : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
   const FastLdsPlan lp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
