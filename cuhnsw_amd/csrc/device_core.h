@@ -665,29 +665,34 @@ __device__ __forceinline__ int frontier_insert(Frontier<NS>& f, float v, uint32_
   bool eq = false;
 #pragma unroll
   for (int j = 0; j < N; ++j) eq = eq || f.k[j] == v;
-  const unsigned long long eq_mask = __ballot(eq);
-  if (eq_mask != 0ull) {
+  const bool any_eq = __ballot(eq) != 0ull;
+  bool dup = false;
+  if (any_eq) {
     bool same = false;
 #pragma unroll
     for (int j = 0; j < N; ++j) same = same || (f.k[j] == v && (f.v[j] & ~kExpanded) == id);
-    if (__ballot(same) != 0ull) return 2;
+    dup = __ballot(same) != 0ull;
   }
-  // last entry of the lane below (lane 0: "-inf", never taken over)
-  const float prev_k = __builtin_bit_cast(
-      float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, f.k[N - 1]), 0x138, 0xF, 0xF, false));
-  const uint32_t prev_v = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f.v[N - 1], 0x138, 0xF, 0xF, false);
-  bool below[N + 1];  // below[j + 1]: v sorts before a[j]; below[0]: before the lane below's last
-  below[0] = v < prev_k;
+  // (one exit: early returns out of an inlined function inside the caller's loops cost the
+  // caller a good deal of scalar control flow)
+  if (!dup) {
+    // last entry of the lane below (lane 0: "-inf", never taken over)
+    const float prev_k = __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, f.k[N - 1]), 0x138, 0xF, 0xF, false));
+    const uint32_t prev_v = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f.v[N - 1], 0x138, 0xF, 0xF, false);
+    bool below[N + 1];  // below[j + 1]: v sorts before a[j]; below[0]: before the lane below's last
+    below[0] = v < prev_k;
 #pragma unroll
-  for (int j = 0; j < N; ++j) below[j + 1] = v < f.k[j];
+    for (int j = 0; j < N; ++j) below[j + 1] = v < f.k[j];
 #pragma unroll
-  for (int j = N - 1; j >= 0; --j) {
-    const float lo_k = j > 0 ? f.k[j - 1] : prev_k;
-    const uint32_t lo_v = j > 0 ? f.v[j - 1] : prev_v;
-    f.k[j] = __builtin_amdgcn_fmed3f(lo_k, v, f.k[j]);
-    f.v[j] = below[j + 1] ? (below[j] ? lo_v : id) : f.v[j];
+    for (int j = N - 1; j >= 0; --j) {
+      const float lo_k = j > 0 ? f.k[j - 1] : prev_k;
+      const uint32_t lo_v = j > 0 ? f.v[j - 1] : prev_v;
+      f.k[j] = __builtin_amdgcn_fmed3f(lo_k, v, f.k[j]);
+      f.v[j] = below[j + 1] ? (below[j] ? lo_v : id) : f.v[j];
+    }
   }
-  return eq_mask != 0ull ? 1 : 0;
+  return dup ? 2 : (any_eq ? 1 : 0);
 }
 template <int NS>
 __device__ __forceinline__ float frontier_max(const Frontier<NS>& f) {
@@ -870,6 +875,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   float group_key = 0.f;
   float group_edge = INFINITY;        // closest key turned away or evicted while the group is expanded
   float ek_min = INFINITY;            // smallest key at which an eviction had equal largest keys to choose from
+  bool gave_up = false;
   while (true) {
     if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
     st.n_dist += n;
@@ -884,30 +890,41 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       unsigned long long todo = __ballot(pass);
       // offers turned away while a group of equal keys is being expanded: remember the closest
       if (exact && in_group) group_edge = uni(fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY)));
+      // (plain if/else nesting, one way out of the loop: `continue` and `return` in here make the
+      // compiler thread a state variable through a dozen scalar blocks per accepted candidate)
       while (todo != 0ull) {
         const int j = __builtin_ctzll(todo);
         todo &= todo - 1ull;
         const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
         const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
-        if (!(st.n_acc < ef || st.lower > key)) {
-          if (exact && in_group) group_edge = uni(fminf(group_edge, key));
-          continue;
+        if (st.n_acc < ef || st.lower > key) {
+          // an eviction out of several equal largest keys: the heap's choice decides which of
+          // them stays in the result set, and the other one stays a live candidate of hnswlib
+          if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = uni(fminf(ek_min, st.lower));
+          const int r = frontier_insert<NS>(fr, key, id, lane);
+          if (r != 2) {
+            have_tie = have_tie || r == 1;
+            if (exact && in_group) {
+              // a closer candidate turning up while a group of equal keys is being expanded would be
+              // expanded before or after the rest of the group depending on the heap's order
+              if (key < group_key) {
+                gave_up = true;
+                todo = 0ull;
+              } else if (st.n_acc >= ef) {
+                group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
+              }
+            }
+            st.n_acc = uni(st.n_acc + 1);
+            st.maxkey = uni(fmaxf(st.maxkey, key));
+            st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
+          }
+        } else if (exact && in_group) {
+          group_edge = uni(fminf(group_edge, key));
         }
-        // an eviction out of several equal largest keys: the heap's choice decides which of
-        // them stays in the result set, and the other one stays a live candidate of hnswlib
-        if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = uni(fminf(ek_min, st.lower));
-        const int r = frontier_insert<NS>(fr, key, id, lane);
-        if (r == 2) continue;
-        have_tie = have_tie || r == 1;
-        // a closer candidate turning up while a group of equal keys is being expanded would be
-        // expanded before or after the rest of the group depending on the heap's order
-        if (exact && in_group && key < group_key) return 1;
-        if (exact && in_group && st.n_acc >= ef) group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
-        st.n_acc = uni(st.n_acc + 1);
-        st.maxkey = uni(fmaxf(st.maxkey, key));
-        st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
       }
+      if (gave_up) base = n;  // leave the outer loop as well
     }
+    if (gave_up) return 1;
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     const int cid = frontier_take<NS>(fr, lane, far);
     if (exact && have_tie) {
