@@ -924,7 +924,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       }
       if (gave_up) base = n;  // leave the outer loop as well
     }
-    if (gave_up) return 1;
+    if (gave_up) break;
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     const int cid = frontier_take<NS>(fr, lane, far);
     if (exact && have_tie) {
@@ -932,30 +932,29 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       if (in_group && d != group_key) {
         // the group is through.  With another order of its members an offer or an entry whose
         // key equals the bound reached now could have ended up on the other side of it.
-        if (st.n_acc >= ef && group_edge == st.lower) return 1;
+        gave_up = st.n_acc >= ef && group_edge == st.lower;
         in_group = false;
       }
       if (cid >= 0) {
-        if (d >= ek_min) return 1;
+        gave_up = gave_up || d >= ek_min;
         if (!in_group) {
           in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
           group_key = d;
           group_edge = INFINITY;
         }
+      } else {
+        // an entry evicted out of equal largest keys that are still within the bound is one
+        // hnswlib would go on to expand
+        gave_up = gave_up || (st.n_acc >= ef && st.lower >= ek_min);
       }
     }
-    if (cid < 0) {
-      // an entry evicted out of equal largest keys that are still within the bound is one
-      // hnswlib would go on to expand
-      if (exact && st.n_acc >= ef && st.lower >= ek_min) return 1;
-      break;
-    }
+    if (gave_up || cid < 0) break;
     st.n_hops += 1;
     wave_sync();
     n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
     wave_sync();
   }
-  return have_tie ? 2 : 0;
+  return gave_up ? 1 : (have_tie ? 2 : 0);
 }
 
 // hnswlib's level-0 search with the literal candidate queue (which alone decides the order of
@@ -998,23 +997,26 @@ __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec
           if (frontier_insert<NS>(fr, e.key, e.id, lane) != 2) {
             amb = amb || twins;
             if (st.cand_size >= cand_cap || st.n_acc >= s.log_cap) {
-              st.fail = 1;
-              return;
-            }
-            if (lane == 0) s.log[st.n_acc] = e;
-            st.n_acc = uni(st.n_acc + 1);
-            if (st.cand_size < s.cand_lds) {
-              LdsHeap cand_fast{s.cand};
-              coop_push<true>(cand_fast, st.cand_size, e, lane);
+              st.fail = 1;  // (one way out of the loops: see search_level_fast)
+              todo = 0ull;
             } else {
-              coop_push<true>(cand, st.cand_size, e, lane);
+              if (lane == 0) s.log[st.n_acc] = e;
+              st.n_acc = uni(st.n_acc + 1);
+              if (st.cand_size < s.cand_lds) {
+                LdsHeap cand_fast{s.cand};
+                coop_push<true>(cand_fast, st.cand_size, e, lane);
+              } else {
+                coop_push<true>(cand, st.cand_size, e, lane);
+              }
+              st.maxkey = uni(fmaxf(st.maxkey, e.key));
+              st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
             }
-            st.maxkey = uni(fmaxf(st.maxkey, e.key));
-            st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
           }
         }
       }
+      if (st.fail) base = n;
     }
+    if (st.fail) break;
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     int cid = -1;
     if (st.cand_size > 0) {
