@@ -540,34 +540,38 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
       HeapEnt e;
       e.key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
       e.id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
-      if (!(st.top_size < ef || st.lower > e.key)) continue;
-      if (st.cand_size >= cand_cap || (NS > 0 && st.n_acc >= s.log_cap)) {
-        st.fail = 1;
-        return;
-      }
-      if (NS > 0 && lane == 0) s.log[st.n_acc] = e;
-      st.n_acc += 1;
-      // the candidate queue normally fits its LDS share: keep that case on pure LDS
-      // instructions (the split accessor compiles to flat loads)
-      if (st.cand_size < s.cand_lds) {
-        LdsHeap cand_fast{s.cand};
-        coop_push<true>(cand_fast, st.cand_size, e, lane);
-      } else {
-        coop_push<true>(cand, st.cand_size, e, lane);
-      }
-      if (NS > 0) {
-        topkeys_insert<NS>(tk, e.key, lane);
-        st.top_size = st.n_acc < ef ? st.n_acc : ef;
-        st.maxkey = fmaxf(st.maxkey, e.key);
-        st.lower = st.n_acc >= ef ? topkeys_max<NS>(tk) : st.maxkey;  // hnswlib's lowerBound
-      } else {
-        LdsHeap top{s.top};
-        coop_push<false>(top, st.top_size, e, lane);
-        if (st.top_size > ef) coop_pop<false>(top, st.top_size, s.tree, lane);
-        wave_sync();
-        st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
+      // (if/else nesting with one way out of the loops, as in search_level_fast)
+      if (st.top_size < ef || st.lower > e.key) {
+        if (st.cand_size >= cand_cap || (NS > 0 && st.n_acc >= s.log_cap)) {
+          st.fail = 1;
+          todo = 0ull;
+        } else {
+          if (NS > 0 && lane == 0) s.log[st.n_acc] = e;
+          st.n_acc += 1;
+          // the candidate queue normally fits its LDS share: keep that case on pure LDS
+          // instructions (the split accessor compiles to flat loads)
+          if (st.cand_size < s.cand_lds) {
+            LdsHeap cand_fast{s.cand};
+            coop_push<true>(cand_fast, st.cand_size, e, lane);
+          } else {
+            coop_push<true>(cand, st.cand_size, e, lane);
+          }
+          if (NS > 0) {
+            topkeys_insert<NS>(tk, e.key, lane);
+            st.top_size = st.n_acc < ef ? st.n_acc : ef;
+            st.maxkey = fmaxf(st.maxkey, e.key);
+            st.lower = st.n_acc >= ef ? topkeys_max<NS>(tk) : st.maxkey;  // hnswlib's lowerBound
+          } else {
+            LdsHeap top{s.top};
+            coop_push<false>(top, st.top_size, e, lane);
+            if (st.top_size > ef) coop_pop<false>(top, st.top_size, s.tree, lane);
+            wave_sync();
+            st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
+          }
+        }
       }
     }
+    if (st.fail) base = n;
   }
 }
 
