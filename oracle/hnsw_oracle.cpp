@@ -45,8 +45,13 @@
 //                           UNPINNED: it cannot run here and leaves the order
 //                           among equal distances to its warp reduction.
 //   file format ........... pinned by closed-form byte layout fixtures
-//   build ................. quality only (recall vs brute force, graph
-//                           invariants); PARITY UNPINNED against real hnswlib.
+//   select_reference ...... (the reference's SearchHeuristic incl. nn_num, save_remains, new_comer) pinned by
+//                           closed-form point sets, by a brute-force statement of HNSW Alg. 4 on integer
+//                           data and by the invariants that characterise its output
+//                           (tests/test_oracle_heuristic.py)
+//   select_neighbors ...... (hnswlib getNeighborsByHeuristic2, used by the CPU build) pinned the same way
+//   build ................. quality only (recall vs brute force asserted >= 0.95 where it serves as a bar,
+//                           graph invariants); PARITY UNPINNED against real hnswlib.
 //
 // Canonical fp32 distance arithmetic (shared by this oracle and the HIP
 // kernels so that ids are bit-comparable): 64 partial sums, element i goes to
@@ -470,6 +475,53 @@ static void select_neighbors(const Index& ix, MaxQueue& top, size_t M) {
   for (const DistId& r : ret) top.emplace(-r.first, r.second);
 }
 
+// The reference's SearchHeuristic restated in full (cpp/include/cuda_build_kernels.cuh:68-162): HNSW Alg. 4 plus
+// the two n2-style extras and the new_comer shortcut of its reverse-link pass.
+//   cand        candidates of `target`, ascending by their key to the target (the reference drains its heap
+//               into that order, :82-88)
+//   nn_num      the first nn_num picks pass untested (= int(max_m * float(heuristic_coef)), :101,105)
+//   save_remains pruned candidates fill the row from its last slot backwards while slots are left (:140-145)
+//               and the degree becomes min(max_m, |cand|) instead of the number of picks (:160)
+//   new_comer   >= 0: every candidate ahead of the newcomer passes untested, the newcomer itself is tested
+//               against all picks so far, and candidates after an accepted newcomer are tested against the
+//               newcomer alone (:105-106,120-123,135-136); -1 switches that off
+// A candidate c is pruned when its key to the target is strictly greater than its key to a pick (:121,126).
+// Returns the degree; row[0..degree) is the new link list with its keys (slots between the picks and the
+// tail fill are only meaningful with save_remains, where there are none left over).
+static int select_reference(const Index& ix, const std::vector<DistId>& cand, int max_m, int nn_num, bool save_remains,
+                            int new_comer, std::vector<DistId>& row, long long* pair_tests = nullptr) {
+  const int T = (int)cand.size();
+  int head = 0;
+  int tail = std::min(max_m, T) - 1;
+  const int max_head = tail + 1;
+  row.assign((size_t)std::max(max_head, 0), DistId(0.0f, 0xFFFFFFFFu));
+  bool inserted = false;
+  for (int j = 0; j < T; ++j) {
+    if (head >= max_m) break;
+    const uint32_t c = cand[j].second;
+    const float to_target = cand[j].first;
+    const bool freepass = head < nn_num || (new_comer >= 0 && !inserted && c != (uint32_t)new_comer);
+    if (freepass) {
+      row[head++] = cand[j];
+      continue;
+    }
+    bool skip = false;
+    if (new_comer >= 0 && inserted) {
+      if (pair_tests) ++*pair_tests;
+      skip = to_target > canon_dist(ix.vec(c), ix.vec((uint32_t)new_comer), ix.D, ix.dist_type);
+    } else {
+      for (int k = 0; k < head && !skip; ++k) {
+        if (pair_tests) ++*pair_tests;
+        skip = to_target > canon_dist(ix.vec(c), ix.vec(row[k].second), ix.D, ix.dist_type);
+      }
+    }
+    if (new_comer >= 0 && c == (uint32_t)new_comer && !skip) inserted = true;
+    if (skip && tail >= head) row[tail--] = cand[j];
+    else if (!skip) row[head++] = cand[j];
+  }
+  return save_remains ? max_head : head;
+}
+
 struct BuildCtx {
   std::vector<std::mutex> locks;
   std::mutex global;
@@ -759,6 +811,33 @@ int orc_select(void* h, const unsigned* cand_ids, const float* cand_d, int n, in
   return (int)v.size();
 }
 
+// the reference's SearchHeuristic on explicit candidates (ascending keys to the target): fills out_ids /
+// out_keys[0..degree) and returns the degree; pair_tests (may be null) receives the number of candidate-pick
+// distance evaluations
+int orc_select_ref(void* h, const unsigned* cand_ids, const float* cand_d, int n, int max_m, int nn_num, int save_remains,
+                   int new_comer, unsigned* out_ids, float* out_keys, long long* pair_tests) {
+  const Index& ix = *static_cast<Index*>(h);
+  std::vector<DistId> cand(n), row;
+  for (int i = 0; i < n; ++i) cand[i] = DistId(cand_d[i], cand_ids[i]);
+  long long tests = 0;
+  const int deg = select_reference(ix, cand, max_m, nn_num, save_remains != 0, new_comer, row, &tests);
+  for (int i = 0; i < deg; ++i) { out_ids[i] = row[i].second; out_keys[i] = row[i].first; }
+  if (pair_tests) *pair_tests = tests;
+  return deg;
+}
+
+// vectors only (no graph): enough for the selection heuristic and for distances by id
+int orc_set_vectors(void* h, const float* vectors, int N, int D, int dist_type) {
+  Index& ix = *static_cast<Index*>(h);
+  ix.N = N; ix.D = D; ix.dist_type = dist_type;
+  ix.vectors.assign(vectors, vectors + (size_t)N * D);
+  ix.levels.assign(N, 0);
+  ix.labels.resize(N);
+  for (int i = 0; i < N; ++i) ix.labels[i] = (uint64_t)i;
+  ix.alloc_links();
+  return 1;
+}
+
 // exact top-k by brute force under the canonical distance; ascending by (distance, id)
 void orc_bruteforce(const float* data, int N, int D, const float* q, int nq, int k, int dist_type, int* ids, float* dists,
                     int threads) {
@@ -795,6 +874,24 @@ int orc_validate(void* h) {
         for (uint32_t b = 0; b < a; ++b) if (ll[1 + b] == x) bad |= 4;
       }
     }
+  return bad;
+}
+
+// level-0 link keys as a builder stored them (N x max_m0, row i = keys of node i's links in list order) against
+// the canonical distance between the two end points: returns the number of links whose stored key differs
+// bitwise (the validator's "stored distance == recomputed distance")
+long long orc_check_link_keys0(void* h, const float* keys0, int threads) {
+  const Index& ix = *static_cast<Index*>(h);
+  long long bad = 0;
+#pragma omp parallel for schedule(static) reduction(+ : bad) num_threads(threads > 0 ? threads : 1)
+  for (int i = 0; i < ix.N; ++i) {
+    const uint32_t* l = ix.list((uint32_t)i, 0);
+    for (uint32_t j = 0; j < l[0]; ++j) {
+      const float d = canon_dist(ix.vec((uint32_t)i), ix.vec(l[1 + j]), ix.D, ix.dist_type);
+      const float got = keys0[(size_t)i * ix.max_m0 + j];
+      if (std::memcmp(&d, &got, 4) != 0) ++bad;
+    }
+  }
   return bad;
 }
 

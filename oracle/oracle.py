@@ -78,6 +78,11 @@ def lib():
                               _c_int_p]
     l.orc_select.argtypes = [ctypes.c_void_p, _c_uint_p, _c_float_p,
                              ctypes.c_int, ctypes.c_int, _c_uint_p]
+    l.orc_select_ref.argtypes = [ctypes.c_void_p, _c_uint_p, _c_float_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                 ctypes.c_int, ctypes.c_int, _c_uint_p, _c_float_p, _c_ll_p]
+    l.orc_set_vectors.argtypes = [ctypes.c_void_p, _c_float_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    l.orc_check_link_keys0.argtypes = [ctypes.c_void_p, _c_float_p, ctypes.c_int]
+    l.orc_check_link_keys0.restype = ctypes.c_longlong
     l.orc_bruteforce.argtypes = [
         _c_float_p, ctypes.c_int, ctypes.c_int, _c_float_p, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _c_int_p, _c_float_p, ctypes.c_int]
@@ -230,6 +235,34 @@ class OracleIndex:
                            _p(cand_dists, _c_float_p), cand_ids.shape[0], m,
                            _p(out, _c_uint_p))
     return out[:n].copy()
+
+  def set_vectors(self, vectors):
+    """Vectors without a graph: enough for select_ref and distances by id."""
+    vectors = _f32(vectors)
+    self._l.orc_set_vectors(self._h, _p(vectors, _c_float_p), vectors.shape[0], vectors.shape[1],
+                            DIST[self.dist_type])
+    return self
+
+  def select_ref(self, cand_ids, cand_keys, max_m, nn_num=0, save_remains=False, new_comer=-1):
+    """The reference's SearchHeuristic on candidates given in ascending order of their key to the
+    target.  Returns (ids, keys, pair_tests): the new link row and how many candidate-pick distances
+    were evaluated."""
+    cand_ids = np.ascontiguousarray(cand_ids, dtype=np.uint32)
+    cand_keys = _f32(cand_keys)
+    out_ids = np.empty(max(max_m, 1), dtype=np.uint32)
+    out_keys = np.empty(max(max_m, 1), dtype=np.float32)
+    tests = ctypes.c_longlong(0)
+    deg = self._l.orc_select_ref(self._h, _p(cand_ids, _c_uint_p), _p(cand_keys, _c_float_p), cand_ids.shape[0],
+                                 max_m, nn_num, int(bool(save_remains)), new_comer, _p(out_ids, _c_uint_p),
+                                 _p(out_keys, _c_float_p), ctypes.byref(tests))
+    return out_ids[:deg].copy(), out_keys[:deg].copy(), tests.value
+
+  def check_link_keys0(self, keys0, threads=None):
+    """Number of level-0 links whose stored key (keys0: N x max_m0) is not bitwise the canonical
+    distance between the link's end points."""
+    keys0 = _f32(keys0)
+    assert keys0.shape == (self.num_data, self.max_m0)
+    return int(self._l.orc_check_link_keys0(self._h, _p(keys0, _c_float_p), threads or host_threads()))
 
   def meets_ties(self, queries, ef_search, threads=None):
     """Per query: does the hnswlib search meet equal distances in its result set?"""
