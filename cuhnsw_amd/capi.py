@@ -16,6 +16,7 @@ SYMBOLS = [
     "cuhnsw_search_knn_device", "cuhnsw_num_data", "cuhnsw_num_dims",
     "cuhnsw_max_level", "cuhnsw_enter_point", "cuhnsw_has_device",
     "cuhnsw_last_build_seconds", "cuhnsw_last_search_repeats", "cuhnsw_set_tunable",
+    "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
 ]
 
 _lib = None
@@ -43,6 +44,8 @@ def load():
   l.cuhnsw_load_index.argtypes = [vp, ctypes.c_char_p]
   l.cuhnsw_search_knn.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp]
   l.cuhnsw_search_knn_device.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp, vp, ctypes.POINTER(ctypes.c_float)]
+  l.cuhnsw_last_build_dropped_links.argtypes = [vp]
+  l.cuhnsw_debug_link_keys0.argtypes = [vp, vp, ctypes.c_longlong]
   for name in ("cuhnsw_num_data", "cuhnsw_num_dims", "cuhnsw_max_level", "cuhnsw_enter_point"):
     getattr(l, name).argtypes = [vp]
   l.cuhnsw_has_device.argtypes = []
@@ -127,6 +130,12 @@ class Engine:
                                                  found_ptr, stats_ptr, ctypes.byref(ms)))
     return ms.value
 
+  def link_keys0(self, max_m0):
+    """Keys stored with the level-0 links by the last build (needs tunable keep_link_keys)."""
+    out = np.empty((self.num_data, max_m0), dtype=np.float32)
+    self._check(self._l.cuhnsw_debug_link_keys0(self._h, out.ctypes.data, out.size))
+    return out
+
   def set_tunable(self, name, value):
     rc = self._l.cuhnsw_set_tunable(self._h, name.encode(), float(value))
     if rc == -2:
@@ -140,3 +149,4 @@ class Engine:
   enter_point = property(lambda s: s._l.cuhnsw_enter_point(s._h))
   last_build_seconds = property(lambda s: s._l.cuhnsw_last_build_seconds(s._h))
   last_search_repeats = property(lambda s: s._l.cuhnsw_last_search_repeats(s._h))
+  last_build_dropped_links = property(lambda s: s._l.cuhnsw_last_build_dropped_links(s._h))

@@ -60,8 +60,17 @@ class CuHNSWBind {
     if ((long long)_nns.size() < (long long)num_queries * topk || (long long)_distances.size() < (long long)num_queries * topk ||
         (long long)_found_cnt.size() < num_queries)
       throw std::runtime_error("output arrays are too small");
-    Check(cuhnsw_search_knn(obj_, _qdata.data(0), num_queries, topk, ef_search, _nns.mutable_data(0),
-                            _distances.mutable_data(0), _found_cnt.mutable_data(0)));
+    const float* q = _qdata.data(0);
+    int* out_nns = _nns.mutable_data(0);
+    float* out_distances = _distances.mutable_data(0);
+    int* out_found = _found_cnt.mutable_data(0);
+    int rc;
+    {
+      // plain pointers from here on: other Python threads may run while the GPU searches
+      py::gil_scoped_release release;
+      rc = cuhnsw_search_knn(obj_, q, num_queries, topk, ef_search, out_nns, out_distances, out_found);
+    }
+    Check(rc);
   }
   // not in the reference: engine facts and tuning knobs
   int NumData() const { return cuhnsw_num_data(obj_); }

@@ -92,6 +92,9 @@ class Engine {
   int fast_path = 1;     // 0: search with the literal queues only; 1: sorted-set pass first when the batch is
                          // larger than one round of literal wavefronts; 2: always
   int last_repeats = 0;  // queries of the last search that were repeated with the literal queues
+  int last_build_dropped = 0;  // reverse links of the last build that found no room in an inbox
+  int keep_link_keys = 0;      // keep the keys stored with the level-0 links after a build (debugging aid)
+  std::vector<float> link_keys0;  // N x max_m0, only with keep_link_keys
   int own_links0 = 0;  // links a new node selects for itself on level 0: 0 = max_m0 (as the reference), else min(value, max_m0); hnswlib uses max_m
   int spill_cap = 0;  // first size of the per-slot queue overflow area (0 = automatic); the accept log is twice that
   int visited_cache = 0;  // entries of the LDS visited cache: 0 = automatic, < 0 = none
@@ -114,13 +117,19 @@ class Engine {
   // staging for the host-pointer search entry point
   DevBuf<float> d_q, d_dist;
   DevBuf<int> d_nns, d_found;
+  long long wall_clock_khz = 100000;        // ticks of wall_clock64() per millisecond
 
   Engine() {
     has_device = device_present();
     if (has_device) {
+      int dev = 0;
+      HIP_CHECK(hipGetDevice(&dev));
       hipDeviceProp_t prop;
-      HIP_CHECK(hipGetDeviceProperties(&prop, 0));
+      HIP_CHECK(hipGetDeviceProperties(&prop, dev));
       num_cus = prop.multiProcessorCount;
+      int khz = 0;
+      if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) == hipSuccess && khz > 0) wall_clock_khz = khz;
+      else (void)hipGetLastError();
       HIP_CHECK(hipStreamCreate(&stream));
       HIP_CHECK(hipEventCreate(&ev0));
       HIP_CHECK(hipEventCreate(&ev1));
@@ -143,14 +152,7 @@ class Engine {
     if (!has_device) throw std::runtime_error("no HIP device available: this call needs a GPU");
   }
 
-  static int padded_dims(int D) { return (D + 31) / 32 * 32; }
-  int qr() const {
-    int chunks16 = ((Dp >> 2) + 15) / 16;
-    if (chunks16 <= 1) return 1;
-    if (chunks16 <= 2) return 2;
-    if (chunks16 <= 4) return 4;
-    return 0;
-  }
+  int qr() const { return query_regs(Dp); }
 
   DevIndex dev_index(float* dists0 = nullptr, float* distsU = nullptr) const {
     DevIndex ix;
@@ -173,11 +175,13 @@ class Engine {
   int init(const char* path) {
     Options o;
     int dt = DIST_DOT;
-    int rc = load_options(path ? path : "", o, dt);
+    std::string why;
+    int rc = load_options(path ? path : "", o, dt, why);
     if (rc == 0) {
       opt = o;
       dist_type = dt;
     }
+    err = why;  // empty after a successful call
     return rc;
   }
 
@@ -371,9 +375,13 @@ class Engine {
     a.live = 0;
     a.nq_total = a.nq;
     a.slot_base = 0;
-    a.spin_limit = spin_limit_override >= 0
-                       ? spin_limit_override
-                       : (int)std::min<long long>(1 << 20, std::max<long long>(1 << 14, (long long)a.nq * 8));  // about 10 us each
+    // a literal wavefront beside the first pass waits at most 2 ms for that pass to start (it is launched
+    // microseconds later unless something serialises the two streams) and accepts no progress of a
+    // started first pass for 100 ms (its queries finish every few microseconds)
+    a.spin_limit = spin_limit_override;
+    a.start_ticks = 2 * wall_clock_khz;
+    a.stall_ticks = 100 * wall_clock_khz;
+    a.nq_dev = nullptr;
     last_repeats = 0;
     HIP_CHECK(hipEventRecord(ev0, stream));
     // the literal pass runs on the sorted set with ids and the LDS filter (no bitmap) unless the
@@ -463,6 +471,9 @@ class Engine {
         if (!answered) {
           scrub_pool();
           if (ctl[1] & 1) glob_cap *= 4;
+          // the wait ran out on its own bound: the streams of this process do not run side by side
+          // (a profiler collecting counters, a saturated device); from now on one pass after the other
+          if ((ctl[1] & 2) && spin_limit_override < 0) concurrent_literal = 0;
         }
       }
     }
@@ -600,8 +611,10 @@ class Engine {
 
     BuildArgs a{};
     a.efc = efc;
-    a.nn_num0 = (int)(host.max_m0 * opt.heuristic_coef);
-    a.nn_numU = (int)(host.max_m * opt.heuristic_coef);
+    // (the reference multiplies in single precision: `const int nn_num = max_m * heuristic_coef` with a
+    // float coefficient, cpp/include/cuda_build_kernels.cuh:77,101)
+    a.nn_num0 = (int)((float)host.max_m0 * (float)opt.heuristic_coef);
+    a.nn_numU = (int)((float)host.max_m * (float)opt.heuristic_coef);
     a.save_remains = opt.save_remains ? 1 : 0;
     a.reverse = opt.reverse_cand ? 1 : 0;
     a.own_cap0 = own_links0 > 0 ? std::min(own_links0, host.max_m0) : host.max_m0;
@@ -612,6 +625,7 @@ class Engine {
     a.inboxU = d_inboxU.p; a.inboxU_cnt = d_inboxU_cnt.p;
     a.cap_in = cap_in;
     a.dirty = d_dirty.p; a.dirty_cnt = d_ctl.p + 2;
+    a.dropped = d_ctl.p + 3;
     const int s_max = std::max(host.S0, host.SU);
     a.lcap = (std::max(s_max, 64) + 63) / 64 * 64;
     size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_max * 8 + 64 +
@@ -623,7 +637,7 @@ class Engine {
     a.cand_lds = sorted_set ? 0 : auto_cand_lds(efc, NS, 64, fixed);
     a.vc_bits = sorted_set ? 0 : auto_vc_bits();
     const LdsPlan lp1 = plan_lds(QR, Dp, sorted_set ? -1 : efc, a.cand_lds, a.lcap, efc, m_max, a.vc_bits, a.fc_bits);
-    const LdsPlan lp3 = plan_lds(QR, Dp, s_max + cap_in, 0, a.lcap, s_max + cap_in, m_max);
+    const LdsPlan lp3 = plan_lds(QR, Dp, s_max + cap_in, 0, a.lcap, s_max + cap_in, std::max(m_max, cap_in));
     const int slots1 = resident_slots(k_search, lp1.total);
     const int slots3 = resident_slots(k_reverse, lp3.total);
     // the sorted-set search needs no per-wavefront global memory (no bitmap, no undo list, no log)
@@ -668,6 +682,16 @@ class Engine {
     if (ctl[1] != 0) {
       scrub_pool();
       throw std::runtime_error("build_graph: candidate queue overflow");
+    }
+    last_build_dropped = ctl[3];
+    if (keep_link_keys) {
+      // debugging aid: the key stored with every level-0 link, for a validator to recompute
+      std::vector<float> strided((size_t)N * host.S0);
+      HIP_CHECK(hipMemcpyAsync(strided.data(), d_dists0.p, strided.size() * 4, hipMemcpyDeviceToHost, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+      link_keys0.assign((size_t)N * host.max_m0, 0.f);
+      for (int i = 0; i < N; ++i)
+        std::memcpy(&link_keys0[(size_t)i * host.max_m0], &strided[(size_t)i * host.S0], (size_t)host.max_m0 * 4);
     }
   }
 
@@ -781,10 +805,7 @@ const char* cuhnsw_last_error(cuhnsw_engine* e) { return e ? e->impl.err.c_str()
 
 int cuhnsw_init(cuhnsw_engine* e, const char* opt_path) {
   if (!e) return -1;
-  int rc = e->impl.init(opt_path);
-  if (rc == 1) e->impl.err = std::string("cannot read or parse option file: ") + (opt_path ? opt_path : "(null)");
-  if (rc == 2) e->impl.err = "invalid dist type " + e->impl.opt.dist_type;
-  return rc;
+  return e->impl.init(opt_path);
 }
 int cuhnsw_set_data(cuhnsw_engine* e, const float* data, int num_data, int num_dims) {
   return guarded(e, [&](Engine& g) { g.set_data(data, num_data, num_dims); });
@@ -812,6 +833,14 @@ int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_que
     g.search_device(d_qdata, num_queries, topk, ef_search, d_nns, d_distances, d_found_cnt, d_stats, kernel_ms);
   });
 }
+int cuhnsw_last_build_dropped_links(cuhnsw_engine* e) { return e ? e->impl.last_build_dropped : 0; }
+int cuhnsw_debug_link_keys0(cuhnsw_engine* e, float* out, long long capacity) {
+  return guarded(e, [&](Engine& g) {
+    if (g.link_keys0.empty()) throw std::runtime_error("link keys were not kept: set tunable keep_link_keys before build_graph");
+    if (!out || capacity < (long long)g.link_keys0.size()) throw std::runtime_error("link keys: output buffer too small");
+    std::memcpy(out, g.link_keys0.data(), g.link_keys0.size() * sizeof(float));
+  });
+}
 int cuhnsw_num_data(cuhnsw_engine* e) { return e ? e->impl.host.N : 0; }
 int cuhnsw_num_dims(cuhnsw_engine* e) { return e ? e->impl.host.D : 0; }
 int cuhnsw_max_level(cuhnsw_engine* e) { return e ? e->impl.host.maxlevel : 0; }
@@ -835,6 +864,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "literal_spin_limit") e->impl.spin_limit_override = (int)value;
   else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(0, std::min(8, (int)value));
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
+  else if (n == "keep_link_keys") e->impl.keep_link_keys = value != 0.0;
   else if (n == "fp16_storage") {
     if (e->impl.have_data && e->impl.storage_half != (value != 0.0)) return -2;  // only before the vectors are there
     e->impl.storage_half = value != 0.0;

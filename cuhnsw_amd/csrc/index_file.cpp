@@ -8,6 +8,7 @@
 #include <cstring>
 #include <memory>
 #include <stdexcept>
+#include <string>
 
 namespace cuhnsw_amd {
 
@@ -165,6 +166,13 @@ void read_index_file(HostIndex& ix, const std::string& path) {
     uint32_t word;
     std::memcpy(&word, rec.data(), 4);
     uint32_t deg = word & 0xffffu;  // hnswlib keeps the count in the low 16 bits, flags above
+    // hnswlib's markDelete sets bit 0 of the word's third byte.  A deleted element is still walked through
+    // by hnswlib's search but never returned, which this engine's search does not reproduce: refuse the
+    // file rather than hand deleted elements back as results (the reference reads the word as a plain
+    // count, cpp/src/cuhnsw_base.cu:311-312, and would index out of its rows).
+    if (word & 0x00010000u)
+      throw std::runtime_error("index file: element " + std::to_string(i) +
+                               " is marked deleted (hnswlib markDelete); files with deleted elements are not supported");
     if (deg > (uint32_t)ix.max_m0) throw std::runtime_error("index file: link count above max_m0");
     uint32_t* row = &l0[(size_t)i * S0];
     std::memcpy(row, rec.data() + 4, (size_t)deg * 4);

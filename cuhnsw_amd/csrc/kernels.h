@@ -49,11 +49,18 @@ struct SearchArgs {
   int* status;   // set to 1 when a candidate queue ran out of room
   int* repeats;  // counts the queries that met equal keys in the sorted-set pass
   int* redo;     // their indices, for the literal pass; as input of the literal pass: the queries to answer (null = all)
-  int* done;     // queries the sorted-set pass has finished with (answered or given up)
+  int* done;     // queries the sorted-set pass has finished with (answered or given up); done[1] is set to 1
+                 // by the first wavefront of that pass to start
   int live;      // literal pass only: 1 = the sorted-set pass is running at the same time and a.redo is
                  // still being filled (entries start at -1); a.nq_total queries will pass through it
   int nq_total;
-  int spin_limit;  // polls of a live literal wavefront before it gives up and reports status 2
+  int spin_limit;  // >= 0: polls of a live literal wavefront before it leaves with status 2 (tests force the
+                   // fall-back with 0); < 0: no bound in polls, the two bounds in time below apply
+  long long start_ticks;  // ticks of the device's wall clock a live literal wavefront waits for the first
+                          // pass to START (done[1] != 0) before it takes the streams to be serialised
+  long long stall_ticks;  // and for which it accepts no progress of the first pass once that has started
+  const int* nq_dev;      // literal pass: when set, the number of list entries is read from here on the
+                          // device (the count the first pass left) instead of taken from nq
   int slot_base;   // first slot of the pool this launch may use (two literal launches can be in flight)
   SlotPool pool;
   int cand_lds, lcap, hnswlib_dist;
@@ -89,9 +96,19 @@ struct BuildArgs {
   int cap_in;
   unsigned long long* dirty;  // node | level << 32
   int* dirty_cnt;
+  int* dropped;  // reverse links that found no room in an inbox (kept: the cap_in closest newcomers)
 };
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
+
+// elements per stored row: D rounded up so that every fp32 row starts on a 128-byte line
+inline int padded_dims(int D) { return (D + 31) / 32 * 32; }
+// float4 registers per lane that hold a query of Dp elements spread over 16 lanes (template parameter QR
+// of the kernels); 0 = the query does not fit registers and is staged in LDS
+inline int query_regs(int Dp) {
+  const int chunks16 = ((Dp >> 2) + 15) / 16;
+  return chunks16 <= 1 ? 1 : (chunks16 <= 2 ? 2 : (chunks16 <= 4 ? 4 : 0));
+}
 
 // LDS layout of one wavefront (shared by host sizing and device carving).  In the build's
 // search kernel the visited filter of the sorted-set search (fcache) takes the place of the
@@ -169,6 +186,8 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   s.nbuf = reinterpret_cast<uint32_t*>(smem + lp.nbuf);
   s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
+  // tells a literal pass waiting beside this one that the two kernels do run at the same time
+  if (blockIdx.x == 0 && lane == 0) __hip_atomic_store(a.done + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   for (;;) {
     int qi = 0;
@@ -282,10 +301,15 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
       if (a.live) {
         // entry qi of the list appears once the sorted-set pass has given up that many
         // queries; it never will if that pass has finished them all and the entry is still
-        // empty.  The wait is bounded: past spin_limit polls the wavefront leaves with
-        // status 2 and the host answers the rest after the first pass.
+        // empty.  The wait is bounded in wall-clock time: if the first pass has not even started
+        // after start_ticks (the two streams are being serialised, as under a counter-collecting
+        // profiler), or has made no progress for stall_ticks, the wavefront leaves with status 2
+        // and the host answers the rest after the first pass.
         int got = -1;
         if (qi < a.nq_total) {
+          const long long t_begin = wall_clock64();
+          long long t_progress = t_begin;
+          int seen_done = -1;
           // (relaxed agent-scope loads: they read the L2 and, unlike acquire loads, do not
           // invalidate this CU's vector cache on every poll; the list entry is the only thing
           // read from the other pass, and it is read after the count that vouches for it)
@@ -295,14 +319,26 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
           for (int spins = 0;; ++spins) {
             got = __hip_atomic_load(&a.redo[qi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (got >= 0) break;
-            if ((spins & 3) == 3 &&
-                __hip_atomic_load(a.done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= a.nq_total) {
-              got = __hip_atomic_load(&a.redo[qi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-              break;
-            }
-            if (spins >= a.spin_limit) {
+            if (a.spin_limit >= 0 && spins >= a.spin_limit) {
               atomicOr(a.status, 2);
               break;
+            }
+            if ((spins & 3) == 3) {
+              const int done_now = __hip_atomic_load(a.done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              if (done_now >= a.nq_total) {
+                got = __hip_atomic_load(&a.redo[qi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+              }
+              const long long now = wall_clock64();
+              if (done_now != seen_done) {
+                seen_done = done_now;
+                t_progress = now;
+              }
+              const bool started = __hip_atomic_load(a.done + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+              if (started ? (now - t_progress > a.stall_ticks) : (now - t_begin > a.start_ticks)) {
+                atomicOr(a.status, 2);
+                break;
+              }
             }
             if (spins < 16) {
               __builtin_amdgcn_s_sleep(32);
@@ -314,7 +350,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
           }
         }
         qi = got;
-      } else if (qi >= a.nq) {
+      } else if (qi >= (a.nq_dev ? *a.nq_dev : a.nq)) {
         qi = -1;
       } else if (a.redo) {
         qi = a.redo[qi];  // second pass: only the queries the sorted-set pass gave up
@@ -707,6 +743,83 @@ __global__ void __launch_bounds__(256) apply_kernel(DevIndex ix, BuildArgs a) {
   }
 }
 
+// More newcomers chose node y on this level than its inbox holds (a hub of a clustered set, late in a
+// large batch).  Which of them reached the inbox depends on the order of the atomics, so the inbox is
+// not used: the batch's selections are scanned for y and the cap closest newcomers by (key, id) are
+// collected into obox (LDS, cap entries) — the same set in every run.  Returns how many newcomers chose
+// y in all.  Rare; one wavefront reads the whole batch's selection rows.
+__device__ __forceinline__ int gather_overflowed_inbox(const DevIndex& ix, const BuildArgs& a, uint32_t y, int level,
+                                                       HeapEnt* obox, int cap, int lane) {
+  int size = 0, total = 0;
+  for (int base = 0; base < a.count; base += 64) {
+    const int b = base + lane;
+    bool hit = false;
+    float my_key = 0.f;
+    uint32_t my_id = kEmpty;
+    if (b < a.count) {
+      const uint32_t x = (uint32_t)(a.begin + b);
+      const int lx = ix.levels[x];
+      const int top_level = lx < a.cur_max ? lx : a.cur_max;
+      if (level <= top_level) {
+        const uint32_t* ids;
+        const float* keys;
+        int deg;
+        if (level == 0) {
+          ids = a.sel0_ids + (size_t)b * ix.max_m0;
+          keys = a.sel0_keys + (size_t)b * ix.max_m0;
+          deg = a.sel0_cnt[b];
+        } else {
+          const size_t r = (size_t)(ix.upper_off[x] + level - 1);
+          ids = a.selU_ids + r * ix.max_m;
+          keys = a.selU_keys + r * ix.max_m;
+          deg = a.selU_cnt[r];
+        }
+        for (int j = 0; j < deg; ++j) {
+          if (ids[j] == y) {
+            hit = true;
+            my_key = keys[j];
+            my_id = x;
+          }
+        }
+      }
+    }
+    unsigned long long todo = __ballot(hit);
+    total += __popcll(todo);
+    while (todo != 0ull) {
+      const int j = __builtin_ctzll(todo);
+      todo &= todo - 1ull;
+      const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+      const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+      if (size < cap) {
+        if (lane == 0) {
+          obox[size].key = key;
+          obox[size].id = id;
+        }
+        size += 1;
+      } else {
+        // the farthest entry of the list by (key, id) gives way if the newcomer is closer
+        const HeapEnt m = obox[lane < cap ? lane : 0];
+        const bool in = lane < cap;
+        const float far_key = -wave_min(in ? -m.key : INFINITY);
+        const bool at_far = in && m.key == far_key;
+        uint32_t far_id = at_far ? m.id : 0u;
+#pragma unroll
+        for (int sh = 32; sh >= 1; sh >>= 1) {
+          const uint32_t o = (uint32_t)__shfl_xor((int)far_id, sh, 64);
+          far_id = o > far_id ? o : far_id;
+        }
+        const bool closer = key < far_key || (key == far_key && id < far_id);
+        if (closer && at_far && m.id == far_id) {
+          obox[lane].key = key;
+          obox[lane].id = id;
+        }
+      }
+      wave_sync();
+    }
+  }
+  return total;
+}
+
 // Phase 3: one wavefront per (node, level) that received reverse links.
 template <int DT, int QR>
 __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
@@ -716,7 +829,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
   const int m_max = ix.max_m0 > ix.max_m ? ix.max_m0 : ix.max_m;
   const int ncand = s_max + a.cap_in;
   // plan: "top" region holds the merged candidates, sorted_* their ranking
-  const LdsPlan lp = plan_lds(QR, ix.Dp, ncand, 0, a.lcap, ncand, m_max);
+  const LdsPlan lp = plan_lds(QR, ix.Dp, ncand, 0, a.lcap, ncand, m_max > a.cap_in ? m_max : a.cap_in);
   Scratch s;
   s.qlds = reinterpret_cast<float4*>(smem + lp.qlds);
   HeapEnt* cbuf = reinterpret_cast<HeapEnt*>(smem + lp.top);
@@ -744,8 +857,17 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       cnt = a.inboxU_cnt + ry;
       box = a.inboxU + ry * a.cap_in;
     }
-    int nin = *cnt;
-    nin = nin < a.cap_in ? nin : a.cap_in;
+    const int posted = *cnt;
+    int nin = posted < a.cap_in ? posted : a.cap_in;
+    if (posted > a.cap_in) {
+      // (the overflow list takes the LDS of the selection's output rows, which are not in use yet; the
+      // host sizes them for cap_in entries)
+      HeapEnt* obox = reinterpret_cast<HeapEnt*>(smem + lp.out_id);
+      const int total = gather_overflowed_inbox(ix, a, y, level, obox, a.cap_in, lane);
+      if (lane == 0) atomicAdd(a.dropped, total - a.cap_in);
+      box = obox;
+      wave_sync();
+    }
     uint32_t* row = link_row_mut(ix, y, level);
     float* drow = dist_row_mut(ix, y, level);
     // existing links

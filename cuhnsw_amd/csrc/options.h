@@ -79,14 +79,20 @@ inline bool parse_flat_json(const std::string& text, std::map<std::string, std::
   return false;
 }
 
-// 0 ok, 1 unreadable / malformed, 2 invalid dist_type
-inline int load_options(const std::string& path, Options& o, int& dist_type) {
+// 0 ok, 1 unreadable / malformed / out of range, 2 invalid dist_type; `why` receives the reason of a failure
+inline int load_options(const std::string& path, Options& o, int& dist_type, std::string& why) {
   std::ifstream f(path);
-  if (!f.is_open()) return 1;
+  if (!f.is_open()) {
+    why = "cannot read option file: " + path;
+    return 1;
+  }
   std::stringstream ss;
   ss << f.rdbuf();
   std::map<std::string, std::string> kv;
-  if (!parse_flat_json(ss.str(), kv)) return 1;
+  if (!parse_flat_json(ss.str(), kv)) {
+    why = "cannot parse option file: " + path;
+    return 1;
+  }
   auto num = [&](const char* k, double def) {
     auto it = kv.find(k);
     if (it == kv.end() || it->second == "null") return def;
@@ -113,8 +119,19 @@ inline int load_options(const std::string& path, Options& o, int& dist_type) {
   if (it != kv.end()) o.dist_type = it->second;
   if (o.dist_type == "dot") dist_type = DIST_DOT;
   else if (o.dist_type == "l2") dist_type = DIST_L2;
-  else return 2;
-  if (o.max_m < 1 || o.max_m0 < 1 || o.ef_construction < 1) return 1;
+  else {
+    why = "invalid dist type " + o.dist_type;
+    return 2;
+  }
+  // the index file keeps a link count in 16 bits
+  if (o.max_m < 1 || o.max_m0 < 1 || o.max_m > 65535 || o.max_m0 > 65535) {
+    why = "max_m and max_m0 must lie in 1..65535";
+    return 1;
+  }
+  if (o.ef_construction < 1) {
+    why = "ef_construction must be positive";
+    return 1;
+  }
   return 0;
 }
 

@@ -97,6 +97,16 @@ int cuhnsw_enter_point(cuhnsw_engine* e);
 int cuhnsw_has_device(void);
 /* seconds spent inside the last cuhnsw_build_graph (device work, event-timed) */
 double cuhnsw_last_build_seconds(cuhnsw_engine* e);
+/* Reverse links of the last cuhnsw_build_graph that were not considered because more than 32 nodes of one
+ * insertion batch chose the same neighbour on one level; the 32 closest of them (by distance, then id) were,
+ * whatever the order the GPU posted them in, so the built graph does not depend on it.  The reference
+ * has no such limit: it re-runs its heuristic once per reverse link under a lock
+ * (cpp/include/cuda_build_kernels.cuh:294-331).  0 on every benchmark configuration. */
+int cuhnsw_last_build_dropped_links(cuhnsw_engine* e);
+/* Debugging aid: the key (ordering distance) the build stored with every level-0 link, row-major
+ * [num_data x max_m0] in list order, as the reference keeps them in its `distances` array
+ * (cpp/include/cuda_build_kernels.cuh:270-278).  Needs tunable "keep_link_keys" = 1 before build_graph. */
+int cuhnsw_debug_link_keys0(cuhnsw_engine* e, float* out, long long capacity);
 /* number of queries of the last search in which two equal distances met and which were therefore
  * searched a second time with literal hnswlib priority queues (the first pass orders candidates
  * by distance alone, which is exact only without ties; the reference has no such distinction
@@ -121,7 +131,11 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *   "literal_per_cu" wavefronts per CU of that concurrent literal pass (0 = automatic: 1 or 2
  *                   depending on how many queries the previous search handed over)
  *   "literal_spin_limit" polls one of its wavefronts may spend waiting for the first pass before
- *                   it leaves and the host answers the remaining queries afterwards (-1 = automatic)
+ *                   it leaves and the host answers the remaining queries afterwards (-1 = no bound in
+ *                   polls: it leaves when the first pass has not started within 2 ms or stalls for
+ *                   100 ms, and the engine then runs the passes one after the other from then on)
+ *   "keep_link_keys" 1 = keep the keys stored with the level-0 links after build_graph for
+ *                   cuhnsw_debug_link_keys0
  *   "lean_literal"  visited set of the literal-queue pass: 0 = exact bitmap in HBM (one bit per point and
  *                   wavefront), 2 = tag filter in LDS with the sorted set catching repeats, 1 = automatic
  *                   (the bitmap while all bitmaps at work fit the L2 caches; default)

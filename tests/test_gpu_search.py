@@ -242,6 +242,44 @@ def test_overflowing_scratch_areas_are_retried(oracle, tmp_path):
   _check_parity(oracle, ix, e, q, 10, 1200)   # literal-heap path
 
 
+def test_search_on_a_file_with_spare_capacity_and_flag_bits(oracle, tmp_path):
+  """An index file as hnswlib writes it from an index that was not filled up (max_elements >
+  cur_element_count: extra level-0 records of arbitrary content) and with unknown flag bits set above
+  the 16-bit link counts: loaded on the GPU it must answer exactly as the oracle does on the compact
+  file; the same file with one element marked deleted is refused."""
+  import struct
+  n, d = 4000, 20
+  x = gauss_mixture(n, d, seed=31)
+  q = gauss_mixture(100, d, seed=32)
+  levels = _levels(n, 0.4, 33)
+  ix = oracle.OracleIndex("dot").build(x, levels, 8, 16, 40, 0.4)
+  p = str(tmp_path / "compact.idx")
+  ix.save(p)
+  raw = bytearray(open(p, "rb").read())
+  rec = 16 * 4 + 4 + d * 4 + 8
+  spare = 37
+  struct.pack_into("<Q", raw, 8, n + spare)                        # max_elements
+  for i in range(0, n, 3):                                         # flag bits above the count, never the delete mark
+    (word,) = struct.unpack_from("<I", raw, 96 + i * rec)
+    struct.pack_into("<I", raw, 96 + i * rec, word | (1 << 17) | (1 << 30))
+  junk = np.random.default_rng(5).integers(0, 256, spare * rec, dtype=np.uint8).tobytes()
+  body_end = 96 + n * rec
+  hnsw_like = bytes(raw[:body_end]) + junk + bytes(raw[body_end:])
+  p2 = str(tmp_path / "spare.idx")
+  open(p2, "wb").write(hnsw_like)
+  e = _engine(tmp_path, dist_type="dot", max_m=8, max_m0=16)
+  e.load_index(p2)
+  assert e.num_data == n
+  _check_parity(oracle, ix, e, q, 10, 80)
+  marked = bytearray(hnsw_like)
+  (word,) = struct.unpack_from("<I", marked, 96 + 5 * rec)
+  struct.pack_into("<I", marked, 96 + 5 * rec, word | (1 << 16))   # hnswlib's markDelete on element 5
+  open(p2, "wb").write(bytes(marked))
+  with pytest.raises(RuntimeError, match="marked deleted"):
+    e.load_index(p2)
+  _check_parity(oracle, ix, e, q[:20], 10, 80, counters=False)     # the refused load left the resident index alone
+
+
 def test_errors(tmp_path):
   e = _engine(tmp_path)
   e.set_data(np.zeros((8, 4), np.float32))

@@ -16,7 +16,7 @@ from cuhnsw_amd import aux, capi, datasets
 
 def test_library_exports_every_declared_symbol():
   header = open(os.path.join(ROOT, "include", "cuhnsw_amd.h")).read()
-  declared = set(re.findall(r"\b(cuhnsw_[a-z_]+)\s*\(", header))
+  declared = set(re.findall(r"\b(cuhnsw_[a-z0-9_]+)\s*\(", header))
   assert declared == set(capi.SYMBOLS)
   lib = ctypes.CDLL(capi.LIB_PATH)
   for name in declared:
@@ -60,9 +60,18 @@ def test_c_init_error_codes(tmp_path):
   assert e.init(bad) == 1
   path, opt = write_options(tmp_path)
   assert e.init(path) == 0
+  assert e._l.cuhnsw_last_error(e._h) == b""    # a successful call leaves no stale message behind
   opt["dist_type"] = "cosine"  # only dot / l2 reach the engine; anything else is an error there
   json.dump(opt, open(path, "w"))
   assert e.init(path) == 2
+  assert e._l.cuhnsw_last_error(e._h) == b"invalid dist type cosine"   # the offending value, not the previous one
+  opt["dist_type"] = "l2"
+  for key, value in (("max_m", 65536), ("max_m0", 70000), ("max_m", 0), ("ef_construction", 0)):
+    json.dump(dict(opt, **{key: value}), open(path, "w"))   # link counts are 16 bits wide in the index file
+    assert e.init(path) == 1
+    assert b"max_m" in e._l.cuhnsw_last_error(e._h) or b"ef_construction" in e._l.cuhnsw_last_error(e._h)
+  json.dump(dict(opt, max_m=65535, max_m0=65535), open(path, "w"))
+  assert e.init(path) == 0
 
 
 def test_level_stream_is_numpy_legacy_mt19937():

@@ -67,16 +67,63 @@ def test_library_reader_writer_bytes(tmp_path):
 
 
 def test_library_reads_hnswlib_count_word_flags(tmp_path):
-  """hnswlib keeps the link count in the low 16 bits of the count word (the upper bits
-  carry flags such as the delete mark): the reader must mask."""
+  """hnswlib keeps the link count in the low 16 bits of the count word; the bits above are flags.
+  Unknown flag bits are masked off.  Bit 0 of the third byte is hnswlib's delete mark: a deleted
+  element must never come back as a search result, which this engine's search does not implement, so
+  such a file is refused with a message that says why."""
   raw = bytearray(expected_bytes())
-  struct.pack_into("<I", raw, 96, 2 | (1 << 16))
+  struct.pack_into("<I", raw, 96, 2 | (1 << 17) | (1 << 31))
   p, q = str(tmp_path / "a.idx"), str(tmp_path / "b.idx")
   open(p, "wb").write(bytes(raw))
   e = capi.Engine()
   e.load_index(p)
   e.save_index(q)
   assert open(q, "rb").read() == expected_bytes()
+  size_data = 3 * 4 + 4 + 2 * 4 + 8
+  struct.pack_into("<I", raw, 96 + size_data, 2 | (1 << 16))     # node 1 marked deleted
+  open(p, "wb").write(bytes(raw))
+  with pytest.raises(RuntimeError, match="element 1 is marked deleted"):
+    e.load_index(p)
+  assert e.num_data == 3                                          # the failed load left the engine as it was
+  e.save_index(q)
+  assert open(q, "rb").read() == expected_bytes()
+
+
+def spare_capacity_bytes(spare=2):
+  """The 3-node index as hnswlib writes it from an index created with max_elements = 3 + spare:
+  the level-0 block has max_elements records (the unused ones are whatever the allocation held,
+  here a pattern), the upper block one entry per existing element."""
+  good = expected_bytes()
+  size_data = 3 * 4 + 4 + 2 * 4 + 8
+  header = bytearray(good[:96])
+  struct.pack_into("<Q", header, 8, 3 + spare)                    # max_elements; cur_element_count stays 3
+  body = good[96:96 + 3 * size_data]
+  junk = bytes((0xA5 + i) & 0xFF for i in range(spare * size_data))
+  return bytes(header) + body + junk + good[96 + 3 * size_data:]
+
+
+def test_library_reads_files_with_spare_capacity(oracle, tmp_path):
+  """max_elements > cur_element_count (an hnswlib index that was not filled up): the unused records
+  are skipped, and saving writes the compact form."""
+  p, q = str(tmp_path / "spare.idx"), str(tmp_path / "compact.idx")
+  for spare in (1, 2, 1000):
+    open(p, "wb").write(spare_capacity_bytes(spare))
+    e = capi.Engine()
+    e.load_index(p)
+    assert (e.num_data, e.num_dims, e.max_level, e.enter_point) == (3, 2, 1, 1)
+    e.save_index(q)
+    assert open(q, "rb").read() == expected_bytes()
+    ix = oracle.OracleIndex("l2").load(p)                         # the checker reads it the same way
+    assert ix.num_data == 3 and list(ix.links(0, 0)) == [1, 2] and list(ix.labels()) == [10, 11, 12]
+  raw = spare_capacity_bytes(2)
+  open(p, "wb").write(raw[:len(raw) - 30])                        # spare records present, upper block cut short
+  with pytest.raises(RuntimeError, match="truncated"):
+    capi.Engine().load_index(p)
+  header = bytearray(raw)
+  struct.pack_into("<Q", header, 8, 2)                            # max_elements below cur_element_count
+  open(p, "wb").write(bytes(header))
+  with pytest.raises(RuntimeError, match="inconsistent header"):
+    capi.Engine().load_index(p)
 
 
 def test_library_rejects_bad_files(tmp_path):
