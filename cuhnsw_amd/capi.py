@@ -16,7 +16,7 @@ SYMBOLS = [
     "cuhnsw_search_knn_device", "cuhnsw_num_data", "cuhnsw_num_dims",
     "cuhnsw_max_level", "cuhnsw_enter_point", "cuhnsw_has_device",
     "cuhnsw_last_build_seconds", "cuhnsw_last_search_repeats", "cuhnsw_set_tunable",
-    "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
+    "cuhnsw_search_knn_device_noalloc", "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
 ]
 
 _lib = None
@@ -44,6 +44,7 @@ def load():
   l.cuhnsw_load_index.argtypes = [vp, ctypes.c_char_p]
   l.cuhnsw_search_knn.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp]
   l.cuhnsw_search_knn_device.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp, vp, ctypes.POINTER(ctypes.c_float)]
+  l.cuhnsw_search_knn_device_noalloc.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_float)]
   l.cuhnsw_last_build_dropped_links.argtypes = [vp]
   l.cuhnsw_debug_link_keys0.argtypes = [vp, vp, ctypes.c_longlong]
   for name in ("cuhnsw_num_data", "cuhnsw_num_dims", "cuhnsw_max_level", "cuhnsw_enter_point"):
@@ -128,6 +129,13 @@ class Engine:
     ms = ctypes.c_float(0.0)
     self._check(self._l.cuhnsw_search_knn_device(self._h, q_ptr, nq, topk, ef_search, nns_ptr, dist_ptr,
                                                  found_ptr, stats_ptr, ctypes.byref(ms)))
+    return ms.value
+
+  def search_knn_device_noalloc(self, q_ptr, nq, topk, ef_search, nns_ptr, dist_ptr, found_ptr):
+    """The search that allocates nothing (device addresses as ints).  Returns the kernel time in ms."""
+    ms = ctypes.c_float(0.0)
+    self._check(self._l.cuhnsw_search_knn_device_noalloc(self._h, q_ptr, nq, topk, ef_search, nns_ptr, dist_ptr,
+                                                         found_ptr, ctypes.byref(ms)))
     return ms.value
 
   def link_keys0(self, max_m0):

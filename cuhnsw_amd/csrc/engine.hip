@@ -41,6 +41,46 @@ static bool device_present() {
   return n > 0;
 }
 
+// ---- scratch of the entry point that allocates nothing (cuhnsw_search_knn_device_noalloc) ----------
+// Everything the two search kernels need beyond the caller's buffers, at fixed maximum sizes, in one
+// array that lives in the code object: each GPU the library runs on holds its own copy from the moment
+// the code object is loaded there until the process ends.  Host code never uses the array's name as an
+// address (it is a host-side stand-in); the device address is looked up once per device
+// (static_scratch_for_current_device) and handed to the kernels like any other buffer.
+constexpr int kStaticMaxQueries = 131072;  // entries of the list of queries the first pass gives up
+constexpr int kStaticMaxEf = 512;          // the sorted set in registers holds up to 512 entries
+constexpr int kStaticSlots = 128;          // wavefronts of the literal pass
+constexpr int kStaticGlobCap = 4096;       // per wavefront: overflow of its candidate queue beyond the LDS share
+constexpr int kStaticLogCap = 8192;        // per wavefront: log of accepted entries
+struct StaticScratch {
+  int ctl[128];
+  int redo[kStaticMaxQueries];
+  HeapEnt cand_glob[(size_t)kStaticSlots * kStaticGlobCap];
+  HeapEnt log[(size_t)kStaticSlots * kStaticLogCap];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(StaticScratch)];  // 12.5 MB
+
+constexpr int kMaxDevices = 64;
+static StaticScratch* g_static_scratch[kMaxDevices] = {};
+// device address of this device's copy of `scratch`; looked up on first use, then kept
+static StaticScratch* static_scratch_for_current_device() {
+  int dev = 0;
+  HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) throw std::runtime_error("device ordinal beyond the table of static scratch addresses");
+  if (!g_static_scratch[dev]) {
+    void* ptr = nullptr;
+    HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    g_static_scratch[dev] = static_cast<StaticScratch*>(ptr);
+  }
+  return g_static_scratch[dev];
+}
+
+// (a fill kernel rather than hipMemsetAsync: a caller may record the no-allocation search into a HIP graph)
+__global__ void __launch_bounds__(128) fill_ints_kernel(int* p, int n, int value) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = value;
+}
+
 template <typename T>
 struct DevBuf {
   T* p = nullptr;
@@ -117,6 +157,8 @@ class Engine {
   // staging for the host-pointer search entry point
   DevBuf<float> d_q, d_dist;
   DevBuf<int> d_nns, d_found;
+  StaticScratch* static_scratch = nullptr;  // this device's copy (device address)
+  int* h_ctl = nullptr;                     // pinned: control words read back without staging
   long long wall_clock_khz = 100000;        // ticks of wall_clock64() per millisecond
 
   Engine() {
@@ -130,6 +172,8 @@ class Engine {
       int khz = 0;
       if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) == hipSuccess && khz > 0) wall_clock_khz = khz;
       else (void)hipGetLastError();
+      static_scratch = static_scratch_for_current_device();
+      HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_ctl), 64 * sizeof(int), hipHostMallocDefault));
       HIP_CHECK(hipStreamCreate(&stream));
       HIP_CHECK(hipEventCreate(&ev0));
       HIP_CHECK(hipEventCreate(&ev1));
@@ -146,6 +190,7 @@ class Engine {
     if (ev_side1) (void)hipEventDestroy(ev_side1);
     if (stream2) (void)hipStreamDestroy(stream2);
     if (stream) (void)hipStreamDestroy(stream);
+    if (h_ctl) (void)hipHostFree(h_ctl);
   }
 
   void need_device() const {
@@ -383,6 +428,10 @@ class Engine {
     a.stall_ticks = 100 * wall_clock_khz;
     a.nq_dev = nullptr;
     last_repeats = 0;
+    if (use_static) {
+      launch_search_static<DT, QR, NS>(ix, a, ms);
+      return;
+    }
     HIP_CHECK(hipEventRecord(ev0, stream));
     // the literal pass runs on the sorted set with ids and the LDS filter (no bitmap) unless the
     // caller asked for literal queues only, which also means exact evaluation counters
@@ -503,6 +552,66 @@ class Engine {
     HIP_CHECK(hipEventSynchronize(ev1));
     if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
   }
+  // The search of the entry point that allocates nothing: the sorted-set pass over every query, then the
+  // literal pass over the list it left, one after the other on the engine's stream.  The length of the
+  // list stays on the device (the literal kernel reads it there), so nothing is read back in between;
+  // control words, list and the literal wavefronts' queue overflow and log areas live in this device's
+  // copy of the static scratch array.  No hipMalloc, no hipFree, no memset: a fill kernel clears the
+  // control words, the list needs no clearing (the pass after reads only the entries the count vouches
+  // for).  Calls that overlap on one GPU would share the array and race.
+  template <int DT, int QR, int NS>
+  void launch_search_static(const DevIndex& ix, SearchArgs& a, float* ms) {
+    if constexpr (NS > 0) {
+      StaticScratch* sc = static_scratch;
+      a.counter = sc->ctl;
+      a.status = sc->ctl + 1;
+      a.repeats = sc->ctl + 32;
+      a.done = sc->ctl + 64;
+      a.redo = sc->redo;
+      a.fast_path = 2;
+      a.lean = a.fc_bits;  // literal searches keep the LDS filter and the sorted set with ids: no bitmap in HBM
+      auto kernel = search_kernel<DT, QR, NS>;
+      auto fast_kernel = search_fast_kernel<DT, QR, NS>;
+      while (filter_entries <= 0 && a.fc_bits > 9) {  // (as in the allocating search: the filter must not cost occupancy)
+        const int now = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits).total);
+        const int with_half = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits - 1).total);
+        if (with_half * 20 < now * 23) break;
+        --a.fc_bits;
+      }
+      const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
+      const LdsPlan lp = plan_lds(QR, ix.Dp, -1, a.cand_lds, a.lcap, 0, 0, 0, 0, a.lean);
+      const int slots = std::max(1, std::min(resident_slots(fast_kernel, fp.total), a.nq));
+      const int lit_slots = std::max(1, std::min(std::min(resident_slots(kernel, lp.total), kStaticSlots), a.nq));
+      HIP_CHECK(hipEventRecord(ev0, stream));
+      hipLaunchKernelGGL(fill_ints_kernel, dim3(1), dim3(128), 0, stream, sc->ctl, 128, 0);
+      HIP_CHECK(hipGetLastError());
+      hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fp.total, stream, ix, a);
+      HIP_CHECK(hipGetLastError());
+      SearchArgs b = a;
+      b.nq = 0;
+      b.nq_dev = sc->ctl + 32;
+      b.counter = sc->ctl + 96;
+      b.pool = SlotPool{};
+      b.pool.cand_glob = sc->cand_glob;
+      b.pool.cand_glob_cap = kStaticGlobCap;
+      b.pool.log = sc->log;
+      b.pool.log_cap = kStaticLogCap;
+      hipLaunchKernelGGL(kernel, dim3(lit_slots), dim3(64), lp.total, stream, ix, b);
+      HIP_CHECK(hipGetLastError());
+      HIP_CHECK(hipEventRecord(ev1, stream));
+      HIP_CHECK(hipMemcpyAsync(h_ctl, sc->ctl, 33 * sizeof(int), hipMemcpyDeviceToHost, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+      last_repeats = h_ctl[32];
+      if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
+      if (h_ctl[1] != 0)
+        throw std::runtime_error("search_knn (no allocation): a literal search outgrew its share of the static scratch "
+                                 "(candidate queue or accept log); use cuhnsw_search_knn_device for this batch");
+    } else {
+      (void)ix; (void)a; (void)ms;
+      throw std::runtime_error("search_knn (no allocation): ef_search beyond the sorted set's capacity");
+    }
+  }
+
   template <int DT, int QR>
   void launch_search_ns(int ns, const DevIndex& ix, SearchArgs& a, float* ms) {
     switch (ns) {
@@ -523,13 +632,24 @@ class Engine {
     }
   }
 
+  bool use_static = false;  // the running search is the one that allocates nothing
+
   void search_device(const float* d_qdata, int nq, int k, int ef, int* d_nns_out, float* d_dist_out, int* d_found_out,
-                     int* d_stats, float* ms) {
+                     int* d_stats, float* ms, bool no_alloc = false) {
     need_device();
     if (!have_graph) throw std::runtime_error("search_knn: no index (call build_graph or load_index first)");
     if (nq <= 0) return;
     if (k <= 0) throw std::runtime_error("search_knn: topk must be positive");
     ef = std::max(ef, k);
+    use_static = no_alloc;
+    if (no_alloc) {
+      if (nq > kStaticMaxQueries)
+        throw std::runtime_error("search_knn (no allocation): at most " + std::to_string(kStaticMaxQueries) + " queries per call");
+      if (ef > kStaticMaxEf)
+        throw std::runtime_error("search_knn (no allocation): max(topk, ef_search) must not exceed " + std::to_string(kStaticMaxEf));
+      if (auto_fc_bits(ef) == 0)
+        throw std::runtime_error("search_knn (no allocation): the index has too many points for the LDS visited filter");
+    }
     DevIndex ix = dev_index();
     SearchArgs a{};
     a.q = d_qdata; a.nq = nq; a.k = k; a.ef = ef;
@@ -540,7 +660,7 @@ class Engine {
     size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
     const int ns = key_slots(ef);
     a.vc_bits = auto_vc_bits();
-    a.fast_path = fast_suspended ? 0 : fast_path;
+    a.fast_path = no_alloc ? 2 : (fast_suspended ? 0 : fast_path);
     a.reverse = opt.reverse_cand ? 1 : 0;
     if (a.reverse) a.fast_path = 2;  // only the sorted set can expand its farthest entry
     a.fc_bits = (ns > 0 && a.fast_path) ? auto_fc_bits(ef) : 0;
@@ -831,6 +951,12 @@ int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_que
                              float* d_distances, int* d_found_cnt, int* d_stats, float* kernel_ms) {
   return guarded(e, [&](Engine& g) {
     g.search_device(d_qdata, num_queries, topk, ef_search, d_nns, d_distances, d_found_cnt, d_stats, kernel_ms);
+  });
+}
+int cuhnsw_search_knn_device_noalloc(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
+                                     int* d_nns, float* d_distances, int* d_found_cnt, float* kernel_ms) {
+  return guarded(e, [&](Engine& g) {
+    g.search_device(d_qdata, num_queries, topk, ef_search, d_nns, d_distances, d_found_cnt, nullptr, kernel_ms, true);
   });
 }
 int cuhnsw_last_build_dropped_links(cuhnsw_engine* e) { return e ? e->impl.last_build_dropped : 0; }

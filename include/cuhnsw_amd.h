@@ -86,6 +86,23 @@ int cuhnsw_search_knn(cuhnsw_engine* e, const float* qdata, int num_queries, int
 int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
                              int* d_nns, float* d_distances, int* d_found_cnt, int* d_stats, float* kernel_ms);
 
+/* The same search for callers that must not allocate device memory (code recorded into a HIP graph,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * SearchGraph allocates on every call (cpp/src/cuhnsw_build.cu:238-249).  Neither this call nor
+ * anything it runs calls hipMalloc, hipFree or a memset: the scratch memory of its kernels (control
+ * words, the list of queries handed from the first pass to the literal pass, the literal wavefronts'
+ * queue overflow and accept log) is a fixed 12.5 MB array inside the library's code object, one copy per
+ * GPU, held until the process ends.  Limits, each rejected with a message: num_queries <= 131072;
+ * max(topk, ef_search) <= 512; fewer than about 2^26 points (the LDS visited filter's 16-bit tags).  A
+ * literal search that outgrows its share of the array (4096 queued candidates beyond its LDS queue, 8192
+ * accepted entries) makes the call fail; cuhnsw_search_knn_device answers such a batch.  The first pass
+ * always runs (tunables fast_path, concurrent_literal and lean_literal do not apply) and the literal pass
+ * follows it on the same stream.  All calls on one GPU share the array: calls that overlap in time on one
+ * GPU — from several engines or threads — race; serialise them.  Same results as
+ * cuhnsw_search_knn_device, bit for bit. */
+int cuhnsw_search_knn_device_noalloc(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
+                                     int* d_nns, float* d_distances, int* d_found_cnt, float* kernel_ms);
+
 /* Introspection used by bindings, tests and the benchmark (the reference keeps
  * the same facts in private members num_data_, num_dims_, max_level_,
  * enter_point_, cpp/include/cuhnsw.hpp:87-108). */
