@@ -698,6 +698,22 @@ __device__ __forceinline__ int frontier_insert(Frontier<NS>& f, float v, uint32_
   }
   return dup ? 2 : (any_eq ? 1 : 0);
 }
+// The same shift for a key that is known to differ from every key of the set (the caller has looked).
+template <int NS>
+__device__ __forceinline__ void frontier_insert_distinct(Frontier<NS>& f, float v, uint32_t id) {
+  constexpr int N = NS > 0 ? NS : 1;
+  const float prev_k = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, f.k[N - 1]), 0x138, 0xF, 0xF, false));
+  const uint32_t prev_v = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f.v[N - 1], 0x138, 0xF, 0xF, false);
+#pragma unroll
+  for (int j = N - 1; j >= 0; --j) {
+    const float lo_k = j > 0 ? f.k[j - 1] : prev_k;
+    const uint32_t lo_v = j > 0 ? f.v[j - 1] : prev_v;
+    const bool before_this = v < f.k[j], before_lower = v < lo_k;
+    f.k[j] = __builtin_amdgcn_fmed3f(lo_k, v, f.k[j]);
+    f.v[j] = before_this ? (before_lower ? lo_v : id) : f.v[j];
+  }
+}
 template <int NS>
 __device__ __forceinline__ float frontier_max(const Frontier<NS>& f) {
   constexpr int N = NS > 0 ? NS : 1;
@@ -880,10 +896,71 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   float group_edge = INFINITY;        // closest key turned away or evicted while the group is expanded
   float ek_min = INFINITY;            // smallest key at which an eviction had equal largest keys to choose from
   bool gave_up = false;
+  // Nine searches in ten never see two equal keys in their set.  Until the first such pair turns up the
+  // search runs in a loop that carries none of the bookkeeping above — same decisions, half the
+  // instructions per accepted candidate — and only then moves on to the general loop below, at the very
+  // offer that met the equal key (resume_at).
+  int resume_at = -1;
+  if (exact && S <= 64) {
+    bool finished = false;
+    while (true) {
+      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      st.n_dist += n;
+      wave_sync();
+      const int at = lane < n ? lane : 0;
+      const float my_key = lane < n ? s.dbuf[at] : INFINITY;
+      const uint32_t my_id = s.nbuf[at];
+      unsigned long long todo = __ballot(lane < n && (st.n_acc < ef || st.lower > my_key));
+      while (todo != 0ull) {
+        const int j = __builtin_ctzll(todo);
+        todo &= todo - 1ull;
+        const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+        const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+        if (st.n_acc < ef || st.lower > key) {
+          bool eq = false;
+#pragma unroll
+          for (int t = 0; t < (NS > 0 ? NS : 1); ++t) eq = eq || fr.k[t] == key;
+          if (__ballot(eq) == 0ull) {
+            frontier_insert_distinct<NS>(fr, key, id);
+            st.n_acc = st.n_acc + 1;
+            if (st.n_acc < ef) {
+              st.maxkey = uni(fmaxf(st.maxkey, key));
+              st.lower = st.maxkey;
+            } else {
+              st.lower = frontier_max<NS>(fr);  // hnswlib's lowerBound
+            }
+          } else {
+            bool same = false;
+#pragma unroll
+            for (int t = 0; t < (NS > 0 ? NS : 1); ++t) same = same || (fr.k[t] == key && (fr.v[t] & ~kExpanded) == id);
+            if (__ballot(same) == 0ull) {
+              resume_at = j;  // an equal key of another node: the rules for equal keys apply from this offer on
+              todo = 0ull;
+            }
+            // (else: a node met again after the visited filter forgot it; it is in the set already)
+          }
+        }
+      }
+      if (resume_at >= 0) break;
+      st.top_size = st.n_acc < ef ? st.n_acc : ef;
+      const int cid = frontier_take<NS>(fr, lane, false);
+      if (cid < 0) {
+        finished = true;
+        break;
+      }
+      st.n_hops += 1;
+      wave_sync();
+      n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
+      wave_sync();
+    }
+    if (finished) return 0;
+  }
   while (true) {
-    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
-    st.n_dist += n;
-    wave_sync();
+    if (resume_at < 0) {
+      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      st.n_dist += n;
+      wave_sync();
+    }
     for (int base = 0; base < n; base += 64) {
       const int mine = base + lane;
       // unconditional LDS reads at a clamped index, then a select: no exec-mask branches
@@ -892,6 +969,10 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       const uint32_t my_id = s.nbuf[at];
       const bool pass = mine < n && (st.n_acc < ef || st.lower > my_key);
       unsigned long long todo = __ballot(pass);
+      if (resume_at >= 0) {
+        todo &= ~((1ull << resume_at) - 1ull);  // the offers before it have been dealt with (one list of at most 64)
+        resume_at = -1;
+      }
       // offers turned away while a group of equal keys is being expanded: remember the closest
       if (exact && in_group) group_edge = uni(fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY)));
       // (plain if/else nesting, one way out of the loop: `continue` and `return` in here make the

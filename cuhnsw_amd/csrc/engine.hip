@@ -126,6 +126,8 @@ class Engine {
   double last_repeat_share = 0.0;         // its wavefronts per CU
   int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
+  int first_pass_waves = 0;  // wavefronts per CU of the first pass (0 = as many as fit)
+  int pair_path = 1;       // first pass with two queries per wavefront where the shapes allow it (0: one per wavefront)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
   bool storage_half = false;  // vectors live in HBM as fp16 (set before set_data / load_index)
@@ -464,17 +466,29 @@ class Engine {
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
       auto fast_kernel = search_fast_kernel<DT, QR, NS>;
+      // two queries per wavefront where the query fits two float4 registers per lane, a link row fits a
+      // half's 32 lanes and the sorted set fits 32 lanes' registers
+      constexpr bool kPairShape = (QR == 1 || QR == 2) && NS == 2;
+      constexpr int N2 = kPairShape ? 2 * NS : 2;
+      auto pair_kernel = search_pair_kernel<DT, (kPairShape ? QR : 1), N2>;
+      const bool pair = kPairShape && pair_path != 0 && !a.reverse && host.S0 <= 32 && host.SU <= 32 && a.nq > 1;
+      auto fast_lds = [&](int bits) -> size_t {
+        return pair ? plan_pair_lds(a.lcap, bits).total : plan_fast_lds(QR, ix.Dp, a.lcap, bits).total;
+      };
+      auto fast_slots = [&](int bits) -> int {
+        return pair ? resident_slots(pair_kernel, fast_lds(bits)) : resident_slots(fast_kernel, fast_lds(bits));
+      };
       // the filter must not be what limits the wavefronts per CU: half the filter repeats more
       // evaluations but is the faster choice wherever it buys occupancy (10 M x 96, ef = 512,
       // five wavefronts per SIMD by registers: 46.8 ms with 8 KB of filter, 45.2 ms with 4 KB)
       while (filter_entries <= 0 && a.fc_bits > 9) {
-        const int now = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits).total);
-        const int with_half = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits - 1).total);
+        const int now = fast_slots(a.fc_bits);
+        const int with_half = fast_slots(a.fc_bits - 1);
         if (with_half * 20 < now * 23) break;  // less than 15 % more
         --a.fc_bits;
       }
-      const FastLdsPlan fp = plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits);
-      int slots = resident_slots(fast_kernel, fp.total);
+      const size_t fast_lds_bytes = fast_lds(a.fc_bits);
+      int slots = fast_slots(a.fc_bits);
       const bool side = concurrent_literal && max_slots_override <= 0;
       int side_slots = 0;
       // few queries need the literal pass (0.4 % of the 1.18M-point set's): one wavefront per CU
@@ -488,7 +502,8 @@ class Engine {
         slots = std::max(num_cus, slots - num_cus * per_cu);  // leave the literal wavefronts their room
       }
       if (max_slots_override > 0) slots = max_slots_override;
-      slots = std::max(1, std::min(slots, a.nq));
+      if (first_pass_waves > 0) slots = std::min(slots, first_pass_waves * num_cus);
+      slots = std::max(1, std::min(slots, pair ? (a.nq + 1) / 2 : a.nq));
       HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 128 * sizeof(int), stream));
       HIP_CHECK(hipMemsetAsync(d_redo.p, 0xFF, (size_t)a.nq * sizeof(int), stream));
       if (side) {
@@ -502,7 +517,8 @@ class Engine {
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipEventRecord(ev_side1, stream2));
       }
-      hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fp.total, stream, ix, a);
+      if (pair) hipLaunchKernelGGL(pair_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
+      else hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
       HIP_CHECK(hipGetLastError());
       if (side) {
         HIP_CHECK(hipStreamWaitEvent(stream, ev_side1, 0));
@@ -624,6 +640,11 @@ class Engine {
   }
   template <int DT>
   void launch_search_qr(int q, int ns, const DevIndex& ix, SearchArgs& a, float* ms) {
+#ifdef CUHNSW_QUICK_BUILD  // experiments only: one query layout
+    if (q != 1) throw std::runtime_error("quick build: only queries of up to 64 dimensions");
+    launch_search_ns<DT, 1>(ns, ix, a, ms);
+    return;
+#endif
     switch (q) {
       case 1: launch_search_ns<DT, 1>(ns, ix, a, ms); break;
       case 2: launch_search_ns<DT, 2>(ns, ix, a, ms); break;
@@ -827,6 +848,11 @@ class Engine {
   }
   template <int DT>
   void build_qr(int q, int ns) {
+#ifdef CUHNSW_QUICK_BUILD
+    if (q != 1) throw std::runtime_error("quick build: only vectors of up to 64 dimensions");
+    build_ns<DT, 1>(ns);
+    return;
+#endif
     switch (q) {
       case 1: build_ns<DT, 1>(ns); break;
       case 2: build_ns<DT, 2>(ns); break;
@@ -986,6 +1012,8 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "fast_path") e->impl.fast_path = (int)value;
   else if (n == "lean_literal") e->impl.lean_literal = (int)value;
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
+  else if (n == "pair_path") e->impl.pair_path = (int)value;
+  else if (n == "first_pass_waves") e->impl.first_pass_waves = (int)value;
   else if (n == "concurrent_literal") e->impl.concurrent_literal = value != 0.0;
   else if (n == "literal_spin_limit") e->impl.spin_limit_override = (int)value;
   else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(0, std::min(8, (int)value));

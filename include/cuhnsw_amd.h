@@ -118,7 +118,8 @@ double cuhnsw_last_build_seconds(cuhnsw_engine* e);
  * insertion batch chose the same neighbour on one level; the 32 closest of them (by distance, then id) were,
  * whatever the order the GPU posted them in, so the built graph does not depend on it.  The reference
  * has no such limit: it re-runs its heuristic once per reverse link under a lock
- * (cpp/include/cuda_build_kernels.cuh:294-331).  0 on every benchmark configuration. */
+ * (cpp/include/cuda_build_kernels.cuh:294-331).  Sets with hubs reach it: 0 on the 50- and 96-dimensional
+ * benchmark configurations, about 12 600 of 25 million links on the 1 M x 128 integer-valued one. */
 int cuhnsw_last_build_dropped_links(cuhnsw_engine* e);
 /* Debugging aid: the key (ordering distance) the build stored with every level-0 link, row-major
  * [num_data x max_m0] in list order, as the reference keeps them in its `distances` array
@@ -143,6 +144,10 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   batch exceeds one round of resident wavefronts, literal queues for the queries
  *                   that met equal distances (default); 2 = first pass whatever the batch size
  *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
+ *   "pair_path"     1 = the first pass runs two queries per wavefront (32 lanes each) where ef_search is at
+ *                   most 128, the vectors have at most 128 dimensions and max_m, max_m0 at most 32
+ *                   (default); 0 = always one query per wavefront.  Same results either way.
+ *   "first_pass_waves" wavefronts per CU of the first pass (0 = as many as fit, the default)
  *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
  *                   (default), 0 = after it
  *   "literal_per_cu" wavefronts per CU of that concurrent literal pass (0 = automatic: 1 or 2

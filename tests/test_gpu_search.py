@@ -111,6 +111,40 @@ def test_search_parity_on_oracle_built_index(oracle, tmp_path, name, n, d, dist,
     _check_parity(oracle, ix, e, q, k, ef)
 
 
+@pytest.mark.parametrize("name,n,d,dist,max_m,max_m0,kind", [CASES[0], CASES[1], CASES[2], CASES[5], CASES[6]],
+                         ids=[CASES[i][0] for i in (0, 1, 2, 5, 6)])
+def test_two_queries_per_wavefront_equal_one_per_wavefront(oracle, tmp_path, name, n, d, dist, max_m, max_m0, kind):
+  """Small ef_search (up to 128): the first pass runs two queries per wavefront, each on half of its lanes.
+  Same answers, same counters and the same queries handed to the literal pass as with one query per
+  wavefront, and both equal to the oracle — odd and even batch sizes, a batch of one, tie-heavy data."""
+  x = _data(kind, n, d, 1)
+  q = _data(kind, 333, d, 2)
+  mult = 1.0 / np.log(max_m)
+  ix = oracle.OracleIndex(dist).build(x, _levels(n, mult, 3), max_m, max_m0, 60, mult)
+  p = str(tmp_path / "i.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=max_m0)
+  e.load_index(p)
+  e.set_tunable("fast_path", 2)
+  for nq, k, ef in ((333, 10, 64), (332, 1, 1), (1, 10, 40), (2, 10, 128), (333, 100, 100), (333, 128, 128), (77, 5, 17)):
+    o_ids, o_d, o_f, o_cnt = ix.search(q[:nq], k, ef, counters=True)
+    got = {}
+    for pair in (1, 0):
+      e.set_tunable("pair_path", pair)
+      got[pair] = _device_search(e, q[:nq], k, ef) + (e.last_search_repeats,)
+      g_ids, g_d, g_f, stats, _ = got[pair]
+      assert (g_f == o_f).all()
+      for r in range(nq):
+        f = o_f[r]
+        assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d pair_path %d k %d ef %d" % (r, pair, k, ef)
+        assert (g_d[r, :f] == o_d[r, :f]).all()
+      assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
+    # evaluation counts too, and the same queries handed over (unless the engine has stopped trying the
+    # first pass on this index because most of its queries tie, which makes the second run literal-only)
+    assert (got[0][3] == got[1][3]).all() and (got[0][4] == got[1][4] or got[0][4] == 0)
+  e.set_tunable("pair_path", 1)
+
+
 def test_labels_from_file_are_returned(oracle, tmp_path):
   n, d = 3000, 20
   x = gauss_mixture(n, d, seed=4)
