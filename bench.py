@@ -17,6 +17,9 @@ measured with HIP events on the engine's stream; `cpu_baseline` times the CPU or
 this host's cores.
 """
 import argparse
+import csv
+import glob
+import hashlib
 import json
 import os
 import sys
@@ -27,6 +30,78 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ["device_core.h", "heap_coop.h", "kernels.h", "pair_search.h", "engine.hip"]
+
+
+def kernel_source_digest():
+  """Digest of the kernel sources: a traffic figure measured on other kernels is not reported."""
+  h = hashlib.sha256()
+  for name in KERNEL_SOURCES:
+    with open(os.path.join(ROOT, "cuhnsw_amd", "csrc", name), "rb") as f:
+      h.update(f.read())
+  return h.hexdigest()[:16]
+
+
+def ingest_pmc(fetch_dir, write_dir, workload):
+  """Turns two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE; both with
+  --profile --copy-calibration) into profiles/hbm_traffic.json: HBM bytes of one search of the
+  batch = the counters summed over the search kernels' dispatches, divided by the number of searches,
+  each scaled by what the same counter reads for the 256 MiB device copy of the calibration."""
+  def read(directory, counter):
+    files = glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)
+    if not files:
+      raise SystemExit("no counter_collection.csv under " + directory)
+    search, first_pass, copies = 0.0, 0, []
+    for row in csv.DictReader(open(files[0])):
+      if row["Counter_Name"] != counter:
+        continue
+      name, value = row["Kernel_Name"], float(row["Counter_Value"])
+      if "cuhnsw_amd::search_" in name:
+        search += value
+        first_pass += ("search_fast_kernel" in name or "search_pair_kernel" in name)
+      elif "copyBuffer" in name:
+        copies.append(value)
+    if not first_pass or not copies:
+      raise SystemExit("%s: no first-pass dispatches or no calibration copy in %s" % (counter, files[0]))
+    return search / first_pass, max(copies), first_pass
+  copy_bytes = 256 * 1024 * 1024
+  fetch, copy_fetch, n_f = read(fetch_dir, "FETCH_SIZE")
+  write, copy_write, n_w = read(write_dir, "WRITE_SIZE")
+  out = {
+      "workload": workload,
+      "kernel_source_digest": kernel_source_digest(),
+      "fetch_size_per_search": fetch, "write_size_per_search": write,
+      "fetch_size_of_256MiB_copy": copy_fetch, "write_size_of_256MiB_copy": copy_write,
+      "searches_counted": [n_f, n_w],
+      "hbm_bytes_per_search": int(fetch * copy_bytes / copy_fetch + write * copy_bytes / copy_write),
+      "fetch_bytes_per_search": int(fetch * copy_bytes / copy_fetch),
+      "write_bytes_per_search": int(write * copy_bytes / copy_write),
+  }
+  with open(TRAFFIC_JSON, "w") as f:
+    json.dump(out, f, indent=1)
+    f.write("\n")
+  print(json.dumps(out))
+
+
+def measured_traffic(workload):
+  """HBM bytes per search from profiles/hbm_traffic.json if it was measured on this workload with these
+  kernel sources; else None."""
+  try:
+    with open(TRAFFIC_JSON) as f:
+      t = json.load(f)
+  except (OSError, ValueError):
+    return None
+  if t.get("workload") != workload or t.get("kernel_source_digest") != kernel_source_digest():
+    return None
+  return t.get("hbm_bytes_per_search")
+
+
+def workload_text(name, n, d, o, nq, k, ef, storage):
+  return "%s: %dx%d %s max_m=%d max_m0=%d ef_construction=%d; %d queries topk=%d ef_search=%d" % (
+      name, n, d, o["dist_type"], o["max_m"], o["max_m0"], o["ef_construction"], nq, k, ef) + (
+          "; vectors stored as fp16 (recall is against the exact neighbours of the unrounded vectors)"
+          if storage == "fp16" else "")
 
 
 def main():
@@ -44,7 +119,30 @@ def main():
                        "to fp16, arithmetic stays fp32 (the default is the configuration the metric is quoted on)")
   ap.add_argument("--copy-calibration", action="store_true",
                   help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+  ap.add_argument("--fast-path", type=int, default=1, choices=[0, 1, 2],
+                  help="0 = literal priority queues only, 1 = default, 2 = sorted-set first pass whatever the batch size")
+  ap.add_argument("--pair-path", type=int, default=1, choices=[0, 1],
+                  help="0 = never two queries per wavefront in the first pass")
+  ap.add_argument("--no-large", action="store_true", help="skip the extra 4x batch (profiling runs)")
+  ap.add_argument("--profile", action="store_true",
+                  help="profiling run: only searches of the default path are launched (no literal-only counting pass, "
+                       "no CPU baseline, no 4x batch); per_query and roofline then use the evaluations performed")
+  ap.add_argument("--tight-rows", action="store_true",
+                  help="vector rows padded to 16-byte chunks only instead of 128-byte lines (layout experiment)")
+  ap.add_argument("--ingest-pmc", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                  help="no benchmark: write profiles/hbm_traffic.json from two rocprofv3 --pmc output directories")
   args = ap.parse_args()
+  if args.profile:
+    args.no_cpu = args.no_large = True
+  if args.ingest_pmc:
+    from cuhnsw_amd import datasets
+    spec = datasets.CONFIGS[args.workload]
+    k = spec["topk"]
+    ef = max(args.ef or (300 if args.workload == "C2" else spec["ef"][-1]), k)
+    ingest_pmc(args.ingest_pmc[0], args.ingest_pmc[1],
+               workload_text(args.workload, args.n or spec["n"], spec["d"], spec["opt"], args.nq or spec["nq"], k, ef,
+                             args.storage))
+    return
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     print("bench.py: this build runs on ONE GPU (the index and the query batch live on a single "
           "device; there is no multi-GPU path) — run with --gpus 1", file=sys.stderr)
@@ -79,14 +177,20 @@ def main():
   assert eng.init(opt_path) == 0
   if args.storage == "fp16":
     eng.set_tunable("fp16_storage", 1)
+  if args.tight_rows:
+    eng.set_tunable("tight_rows", 1)
   t0 = time.time()
   eng.set_data(data)
   upload_s = time.time() - t0
+  eng.set_tunable("build_counters", 1)
   eng.set_random_levels(levels)
-  eng.build_graph()                      # warm-up build (first launch pays code loading)
+  eng.build_graph()                      # warm-up build (first launch pays code loading); its work is counted
+  build_work = eng.build_counters()
+  eng.set_tunable("build_counters", 0)
   eng.set_random_levels(levels)
-  eng.build_graph()
+  eng.build_graph()                      # the timed build (same graph: the build is deterministic)
   build_s = eng.last_build_seconds
+  eng.set_tunable("pair_path", args.pair_path)
 
   # exact top-k on the GPU (harness only) for recall.  Scores are produced in blocks of at most
   # 2^28 elements (1 GiB): larger matmul outputs came back with wrong entries on this stack.
@@ -126,12 +230,16 @@ def main():
   # algorithmic counters (distinct evaluations, expansions) come from a pass with the literal
   # queues only; the timed default path may evaluate a node again after its visited filter
   # has forgotten it, and those repeats must not count as useful bytes
-  eng.set_tunable("fast_path", 0)
-  step(with_stats=True)
-  st = stats.cpu().numpy().astype(np.int64)
-  eng.set_tunable("fast_path", 1)
+  eng.set_tunable("fast_path", args.fast_path)
   step(with_stats=True)
   st_run = stats.cpu().numpy().astype(np.int64)
+  st = st_run
+  if not args.profile:
+    eng.set_tunable("fast_path", 0)
+    step(with_stats=True)
+    st = stats.cpu().numpy().astype(np.int64)
+    eng.set_tunable("fast_path", args.fast_path)
+    step(with_stats=True)
   repeats = eng.last_search_repeats
   for _ in range(args.warmup):
     step()
@@ -156,8 +264,15 @@ def main():
   # the same index with four times the batch (fresh queries of the same law): what the
   # kernels sustain once a launch holds several rounds of wavefronts.  Reported beside the
   # headline figure, never in its place.
+  # the entry point most callers use (host pointers: queries staged to the device, results copied back)
+  t0 = time.perf_counter()
+  for _ in range(5):
+    h_ids, h_d, h_f = eng.search_knn(queries, k, ef)
+  host_ms = (time.perf_counter() - t0) / 5 * 1e3
+  host_equal = bool((h_ids == ids).all())
+
   large = None
-  if args.workload == "C2" and args.n is None and args.nq is None:
+  if args.workload == "C2" and args.n is None and args.nq is None and not args.no_large:
     _, q_large, _ = datasets.make(args.workload, n=1, nq=4 * nq)
     ql = torch.from_numpy(q_large).cuda()
     nl = ql.shape[0]
@@ -171,15 +286,13 @@ def main():
     del ql, l_nns, l_dist, l_found
 
   avg_kernel_ms = float(np.mean(kernel_ms))
+  row_bytes_stored = (2 if args.storage == "fp16" else 4) * d
   gather_bytes = int(st[:, 0].sum()) * (2 if args.storage == "fp16" else 4) * d
-  # HBM bytes of one search of the default batch, measured once with two rocprofv3 --pmc runs of
-  # this very command (FETCH_SIZE 2 009 400 + 7 308 KiB over both search kernels, scaled by 2.0:
-  # a 256 MiB device copy reads 131 084 on that counter; WRITE_SIZE 7 584 + 196 KiB, scaled by
-  # 1.0: the copy writes 262 144).  It cannot be measured from inside this process; other
-  # workloads report null.
-  traffic = None
-  if args.workload == "C2" and args.n is None and args.nq is None and ef == 300 and args.storage == "fp32":
-    traffic = int((2009400 + 7308) * 1024 * 2.0 + (7584 + 196) * 1024 * 1.0)
+  # HBM bytes of one search of the batch: read from profiles/hbm_traffic.json, which `--ingest-pmc` writes from
+  # two rocprofv3 --pmc runs of this script; null when that file was measured on another workload or on
+  # other kernel sources (it cannot be measured from inside this process)
+  wl = workload_text(args.workload, n, d, o, nq, k, ef, args.storage) + ("; rows padded to 16 bytes" if args.tight_rows else "")
+  traffic = measured_traffic(wl) if args.fast_path == 1 and args.pair_path == 1 else None
   achieved = gather_bytes / (avg_kernel_ms * 1e-3) / 1e9
   out = {
       "metric": "batch search QPS at recall@%d (%s: %dx%d %s), with build seconds" % (
@@ -190,10 +303,7 @@ def main():
       "ms_per_step": elapsed / args.steps * 1e3,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
       "dtype": "f32", "data": "synthetic",
-      "config": {"workload": "%s: %dx%d %s max_m=%d max_m0=%d ef_construction=%d; %d queries topk=%d ef_search=%d" % (
-          args.workload, n, d, o["dist_type"], o["max_m"], o["max_m0"], o["ef_construction"], nq, k, ef) + (
-              "; vectors stored as fp16 (recall is against the exact neighbours of the unrounded vectors)"
-              if args.storage == "fp16" else "")},
+      "config": {"workload": wl},
       "build_seconds": build_s,
       "recall_at_k": recall,
       "upload_seconds": upload_s, "datagen_seconds": gen_s,
@@ -204,12 +314,43 @@ def main():
                     "queries_repeated_with_literal_queues": int(repeats)},
       "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                    "frac": achieved / 8000.0, "traffic": traffic,
-                   "kernel": "search_fast_kernel with search_kernel beside it (one search of the batch)",
+                   "kernel": ("search_pair_kernel" if (args.pair_path and ef <= 128 and d <= 128) else "search_fast_kernel") +
+                             " with search_kernel beside it (one search of the batch)"
+                             if args.fast_path else "search_kernel (literal priority queues only)",
                    "algorithmic_bytes_per_launch": gather_bytes},
+      "host_pointer_search": {"ms_per_call": host_ms, "value": nq / (host_ms * 1e-3), "unit": "queries/s",
+                              "same_ids_as_device_pointer_search": host_equal,
+                              "note": "cuhnsw_search_knn: queries staged from pageable host memory, results copied back"},
+  }
+  # build roofline: bytes the build's kernels asked for, from device counters of an identical build
+  row_bytes = (2 if args.storage == "fp16" else 4) * d
+  lv0, up = build_work["level0"], build_work["upper"]
+  s0 = (o["max_m0"] + 31) // 32 * 32 * 4
+  su = (o["max_m"] + 15) // 16 * 16 * 4
+  build_bytes = ((lv0[0] + lv0[2] + lv0[3] + up[0] + up[2] + up[3]) * row_bytes
+                 + (lv0[1] + lv0[4]) * s0 + (up[1] + up[4]) * su)
+  out["build_roofline"] = {
+      "bound": "hbm", "achieved": build_bytes / build_s / 1e9, "peak": 8000.0, "unit": "GB/s",
+      "frac": build_bytes / build_s / 1e9 / 8000.0, "algorithmic_bytes": int(build_bytes),
+      "counters": {"names": ["distance evaluations (searches, descents)", "link rows read", "heuristic pair tests",
+                             "heuristic candidate rows", "link rows written"], "level0": lv0, "upper_levels": up},
+      "note": "vector rows x %d B + link rows x %d B (level 0) / %d B (upper levels), over build_seconds" % (row_bytes, s0, su),
   }
 
   if large:
     out["large_batch"] = large
+
+  # the memory system alone: random gathers of this index's rows, with as many wavefronts per CU as the first
+  # pass holds and as many rows in flight per wavefront as a hop fetches on average (4) and at most (16)
+  probes = []
+  for waves_per_cu, in_flight in ((28, 4), (28, 16), (8, 4)):
+    rows, ms = eng.gather_probe(waves_per_cu, in_flight, True)
+    probes.append({"waves_per_cu": waves_per_cu, "rows_in_flight_per_wavefront": in_flight, "rows_per_s": rows / (ms * 1e-3),
+                   "GB_per_s": rows * row_bytes_stored / (ms * 1e-3) / 1e9,
+                   "us_per_dependent_batch": ms * 1e3 / 2048.0})
+  out["gather_ceiling"] = {"probes": probes, "search_rows_per_s": float(st_run[:, 0].sum()) / (avg_kernel_ms * 1e-3),
+                           "note": "cuhnsw_debug_gather_probe: dependent batches of random row fetches over the resident vectors, "
+                                   "nothing else; search_rows_per_s = evaluations the search performs per second"}
 
   if not args.no_cpu:
     from oracle import oracle as orc

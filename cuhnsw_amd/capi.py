@@ -17,6 +17,7 @@ SYMBOLS = [
     "cuhnsw_max_level", "cuhnsw_enter_point", "cuhnsw_has_device",
     "cuhnsw_last_build_seconds", "cuhnsw_last_search_repeats", "cuhnsw_set_tunable",
     "cuhnsw_search_knn_device_noalloc", "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
+    "cuhnsw_last_build_counters", "cuhnsw_debug_gather_probe",
 ]
 
 _lib = None
@@ -47,6 +48,8 @@ def load():
   l.cuhnsw_search_knn_device_noalloc.argtypes = [vp, vp, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_float)]
   l.cuhnsw_last_build_dropped_links.argtypes = [vp]
   l.cuhnsw_debug_link_keys0.argtypes = [vp, vp, ctypes.c_longlong]
+  l.cuhnsw_last_build_counters.argtypes = [vp, vp, ci]
+  l.cuhnsw_debug_gather_probe.argtypes = [vp, ci, ci, ci, ctypes.POINTER(cd), ctypes.POINTER(ctypes.c_float)]
   for name in ("cuhnsw_num_data", "cuhnsw_num_dims", "cuhnsw_max_level", "cuhnsw_enter_point"):
     getattr(l, name).argtypes = [vp]
   l.cuhnsw_has_device.argtypes = []
@@ -143,6 +146,21 @@ class Engine:
     out = np.empty((self.num_data, max_m0), dtype=np.float32)
     self._check(self._l.cuhnsw_debug_link_keys0(self._h, out.ctypes.data, out.size))
     return out
+
+  def gather_probe(self, waves_per_cu, rows_in_flight, dependent=True):
+    """Random row gathers over the resident vectors alone: returns (rows fetched, kernel ms)."""
+    rows, ms = ctypes.c_double(0.0), ctypes.c_float(0.0)
+    self._check(self._l.cuhnsw_debug_gather_probe(self._h, waves_per_cu, rows_in_flight, int(bool(dependent)),
+                                                  ctypes.byref(rows), ctypes.byref(ms)))
+    return rows.value, ms.value
+
+  def build_counters(self):
+    """Work of the last build counted on the device (needs tunable build_counters): dict of two lists
+    [evaluations, link rows read, heuristic pair tests, heuristic candidate rows, link rows written]."""
+    out = np.zeros(10, dtype=np.uint64)
+    if self._l.cuhnsw_last_build_counters(self._h, out.ctypes.data, 10) != 0:
+      raise RuntimeError("cuhnsw_last_build_counters failed")
+    return {"level0": [int(v) for v in out[:5]], "upper": [int(v) for v in out[5:]]}
 
   def set_tunable(self, name, value):
     rc = self._l.cuhnsw_set_tunable(self._h, name.encode(), float(value))

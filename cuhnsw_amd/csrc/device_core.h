@@ -210,8 +210,8 @@ __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const flo
 
 // one pass over 4*U rows starting at ids[r]: loads first, arithmetic after
 template <int DT, int R, int U, bool RAW, bool HALF>
-__device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, const float4* q, const uint32_t* ids, int r,
-                                          int n, float* out, int g, int sub) {
+__device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, uint32_t used, const float4* q,
+                                          const uint32_t* ids, int r, int n, float* out, int g, int sub) {
   float4 v[U][R];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -221,13 +221,14 @@ __device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, con
 #pragma unroll
     for (int k = 0; k < R; ++k) {
       // always one unconditional load (a guarded one is split into dword loads); a chunk past
-      // the row end re-reads chunk 0.  The query holds zeros there, which is all a dot product
-      // needs (finite data); for L2 the chunk is replaced by the query's own zeros.  Rows are
-      // longer than 16 * (R / 2) chunks, so only the upper half of k can be past the end.
+      // the row's data (`used` chunks; the row's stride may be longer) re-reads chunk 0, which costs no
+      // further memory line.  The query holds zeros there, which is all a dot product needs (finite
+      // data); for L2 the chunk is replaced by the query's own zeros.  The data is longer than
+      // 16 * (R / 2) chunks, so only the upper half of k can be past its end.
       const uint32_t c = sub + 16 * k;
-      const uint64_t at = first + (c < rowlen ? c : 0);
+      const uint64_t at = first + (c < used ? c : 0);
       const float4 t = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
-      v[u][k] = (DT == DIST_DOT || k < R / 2 || c < rowlen) ? t : q[k];
+      v[u][k] = (DT == DIST_DOT || k < R / 2 || c < used) ? t : q[k];
     }
   }
 #pragma unroll
@@ -245,10 +246,10 @@ __device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, con
 // has rowlen/16 chunks to fetch; they are issued eight at a time to keep eight loads per lane
 // in flight, the query chunks come from LDS
 template <int DT, bool RAW, bool HALF>
-__device__ __forceinline__ void dist_long(const void* rows, int rowlen, const float4* qlds, const uint32_t* ids, int n,
-                                          float* out, int g, int sub) {
+__device__ __forceinline__ void dist_long(const void* rows, int rowlen, int used, const float4* qlds, const uint32_t* ids,
+                                          int n, float* out, int g, int sub) {
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-  const int nk = (rowlen + 15) >> 4;
+  const int nk = (used + 15) >> 4;
   constexpr int B = 8;
   for (int r = 0; r < n; r += 4) {
     const int idx = r + g;
@@ -260,9 +261,9 @@ __device__ __forceinline__ void dist_long(const void* rows, int rowlen, const fl
 #pragma unroll
       for (int b = 0; b < B; ++b) {
         const int c = sub + 16 * (k0 + b);
-        const uint64_t at = first + (c < rowlen ? c : 0);  // unconditional load
+        const uint64_t at = first + (c < used ? c : 0);  // unconditional load
         const float4 t = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
-        v[b] = c < rowlen ? t : zero;
+        v[b] = c < used ? t : zero;
       }
 #pragma unroll
       for (int b = 0; b < B; ++b) {
@@ -283,6 +284,7 @@ __device__ __forceinline__ void dist_list_t(const DevIndex& ix, const QVec<QR>& 
                                             int n, float* out, int lane) {
   const int g = lane >> 4, sub = lane & 15;
   const int rowlen = ix.Dp >> 2;
+  const int used = (ix.D + 3) >> 2;  // chunks of a row that hold data
   const void* rows = ix.vectors;
   if (QR > 0) {
     constexpr int R = QR > 0 ? QR : 1;
@@ -291,18 +293,18 @@ __device__ __forceinline__ void dist_list_t(const DevIndex& ix, const QVec<QR>& 
     while (r < n) {
       const int rem = n - r;
       if (UMAX >= 4 && rem > 8) {
-        dist_pass<DT, R, (UMAX >= 4 ? 4 : 1), RAW, HALF>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        dist_pass<DT, R, (UMAX >= 4 ? 4 : 1), RAW, HALF>(rows, rowlen, used, qv.q, ids, r, n, out, g, sub);
         r += 16;
       } else if (UMAX >= 2 && rem > 4) {
-        dist_pass<DT, R, (UMAX >= 2 ? 2 : 1), RAW, HALF>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        dist_pass<DT, R, (UMAX >= 2 ? 2 : 1), RAW, HALF>(rows, rowlen, used, qv.q, ids, r, n, out, g, sub);
         r += 8;
       } else {
-        dist_pass<DT, R, 1, RAW, HALF>(rows, rowlen, qv.q, ids, r, n, out, g, sub);
+        dist_pass<DT, R, 1, RAW, HALF>(rows, rowlen, used, qv.q, ids, r, n, out, g, sub);
         r += 4;
       }
     }
   } else {
-    dist_long<DT, RAW, HALF>(rows, rowlen, qlds, ids, n, out, g, sub);
+    dist_long<DT, RAW, HALF>(rows, rowlen, used, qlds, ids, n, out, g, sub);
   }
 }
 // (the element type of the stored vectors is a property of the index: one scalar branch per list)

@@ -131,9 +131,12 @@ class Engine {
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
   bool storage_half = false;  // vectors live in HBM as fp16 (set before set_data / load_index)
+  bool tight_rows = false;    // rows padded to 16-byte chunks only, not to 128-byte lines (set before set_data / load_index)
   int fast_path = 1;     // 0: search with the literal queues only; 1: sorted-set pass first when the batch is
                          // larger than one round of literal wavefronts; 2: always
   int last_repeats = 0;  // queries of the last search that were repeated with the literal queues
+  int count_build_work = 0;    // count the work of a build on the device (cuhnsw_last_build_counters)
+  unsigned long long build_counters[10] = {};
   int last_build_dropped = 0;  // reverse links of the last build that found no room in an inbox
   int keep_link_keys = 0;      // keep the keys stored with the level-0 links after a build (debugging aid)
   std::vector<float> link_keys0;  // N x max_m0, only with keep_link_keys
@@ -237,7 +240,7 @@ class Engine {
   // With fp16 storage the host copy is rounded to the stored values first: everything downstream
   // (the saved file, a CPU search of that file) then sees exactly the vectors the kernels see.
   void upload_vectors() {
-    Dp = padded_dims(host.D);
+    Dp = padded_dims(host.D, tight_rows);
     const size_t n = (size_t)host.N;
     if (storage_half) {
       for (float& x : host.vectors) x = (float)(_Float16)x;
@@ -767,6 +770,12 @@ class Engine {
     a.cap_in = cap_in;
     a.dirty = d_dirty.p; a.dirty_cnt = d_ctl.p + 2;
     a.dropped = d_ctl.p + 3;
+    DevBuf<unsigned long long> d_work;
+    if (count_build_work) {
+      d_work.reserve(10);
+      HIP_CHECK(hipMemsetAsync(d_work.p, 0, 10 * sizeof(unsigned long long), stream));
+    }
+    a.counters = d_work.p;
     const int s_max = std::max(host.S0, host.SU);
     a.lcap = (std::max(s_max, 64) + 63) / 64 * 64;
     size_t fixed = (size_t)a.lcap * 8 + (size_t)efc * 8 + (size_t)m_max * 8 + 64 +
@@ -825,6 +834,11 @@ class Engine {
       throw std::runtime_error("build_graph: candidate queue overflow");
     }
     last_build_dropped = ctl[3];
+    std::memset(build_counters, 0, sizeof(build_counters));
+    if (count_build_work) {
+      HIP_CHECK(hipMemcpyAsync(build_counters, d_work.p, sizeof(build_counters), hipMemcpyDeviceToHost, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+    }
     if (keep_link_keys) {
       // debugging aid: the key stored with every level-0 link, for a validator to recompute
       std::vector<float> strided((size_t)N * host.S0);
@@ -875,6 +889,34 @@ class Engine {
     have_graph = true;
     fast_suspended = false;
     host_links_stale = true;
+  }
+
+  // ---- measurement aid --------------------------------------------------------------------------------
+  // random row gathers over the resident vectors (gather_probe_kernel): returns rows fetched, ms taken
+  void gather_probe(int waves_per_cu, int rows_in_flight, int dependent, double* rows, float* ms) {
+    need_device();
+    if (!have_data) throw std::runtime_error("gather probe: no vectors (call set_data or load_index first)");
+    const int waves = std::max(1, std::min(waves_per_cu, 32)) * num_cus;
+    const int batches = 2048;
+    const int U = rows_in_flight >= 16 ? 4 : (rows_in_flight >= 8 ? 2 : 1);
+    DevBuf<float> sink;
+    sink.reserve((size_t)waves);
+    DevIndex ix = dev_index();
+    float best = 0.f;
+    for (int it = 0; it < 3; ++it) {
+      HIP_CHECK(hipEventRecord(ev0, stream));
+      if (U == 4) hipLaunchKernelGGL(gather_probe_kernel<4>, dim3(waves), dim3(64), 0, stream, ix, batches, dependent, sink.p);
+      else if (U == 2) hipLaunchKernelGGL(gather_probe_kernel<2>, dim3(waves), dim3(64), 0, stream, ix, batches, dependent, sink.p);
+      else hipLaunchKernelGGL(gather_probe_kernel<1>, dim3(waves), dim3(64), 0, stream, ix, batches, dependent, sink.p);
+      HIP_CHECK(hipGetLastError());
+      HIP_CHECK(hipEventRecord(ev1, stream));
+      HIP_CHECK(hipEventSynchronize(ev1));
+      float t = 0.f;
+      HIP_CHECK(hipEventElapsedTime(&t, ev0, ev1));
+      if (it == 0 || t < best) best = t;
+    }
+    if (rows) *rows = (double)waves * 4.0 * U * batches;
+    if (ms) *ms = best;
   }
 
   // ---- index file --------------------------------------------------------------------------------
@@ -985,7 +1027,16 @@ int cuhnsw_search_knn_device_noalloc(cuhnsw_engine* e, const float* d_qdata, int
     g.search_device(d_qdata, num_queries, topk, ef_search, d_nns, d_distances, d_found_cnt, nullptr, kernel_ms, true);
   });
 }
+int cuhnsw_debug_gather_probe(cuhnsw_engine* e, int waves_per_cu, int rows_in_flight, int dependent, double* rows,
+                              float* ms) {
+  return guarded(e, [&](Engine& g) { g.gather_probe(waves_per_cu, rows_in_flight, dependent, rows, ms); });
+}
 int cuhnsw_last_build_dropped_links(cuhnsw_engine* e) { return e ? e->impl.last_build_dropped : 0; }
+int cuhnsw_last_build_counters(cuhnsw_engine* e, unsigned long long* out, int n) {
+  if (!e || !out || n < 10) return -1;
+  std::memcpy(out, e->impl.build_counters, sizeof(e->impl.build_counters));
+  return 0;
+}
 int cuhnsw_debug_link_keys0(cuhnsw_engine* e, float* out, long long capacity) {
   return guarded(e, [&](Engine& g) {
     if (g.link_keys0.empty()) throw std::runtime_error("link keys were not kept: set tunable keep_link_keys before build_graph");
@@ -1019,6 +1070,11 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "literal_per_cu") e->impl.side_per_cu = std::max(0, std::min(8, (int)value));
   else if (n == "spill_cap") e->impl.spill_cap = (int)value;
   else if (n == "keep_link_keys") e->impl.keep_link_keys = value != 0.0;
+  else if (n == "build_counters") e->impl.count_build_work = value != 0.0;
+  else if (n == "tight_rows") {
+    if (e->impl.have_data && e->impl.tight_rows != (value != 0.0)) return -2;  // only before the vectors are there
+    e->impl.tight_rows = value != 0.0;
+  }
   else if (n == "fp16_storage") {
     if (e->impl.have_data && e->impl.storage_half != (value != 0.0)) return -2;  // only before the vectors are there
     e->impl.storage_half = value != 0.0;

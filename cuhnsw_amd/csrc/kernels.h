@@ -98,12 +98,21 @@ struct BuildArgs {
   unsigned long long* dirty;  // node | level << 32
   int* dirty_cnt;
   int* dropped;  // reverse links that found no room in an inbox (kept: the cap_in closest newcomers)
+  // optional work counters of a build (null = off), level 0 in [0..4], upper levels in [5..9]:
+  //   +0 distance evaluations of the searches and descents (one vector row each)
+  //   +1 link rows read (expanded candidates, descent sweeps, rows merged with their inbox)
+  //   +2 pair tests of the selection heuristic (one vector row each)
+  //   +3 candidates the heuristic loaded to test them (one vector row each)
+  //   +4 link rows written
+  unsigned long long* counters;
 };
+
 
 __host__ __device__ inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 
-// elements per stored row: D rounded up so that every fp32 row starts on a 128-byte line
-inline int padded_dims(int D) { return (D + 31) / 32 * 32; }
+// elements per stored row: D rounded up so that every fp32 row starts on a 128-byte line (32 elements), or —
+// `tight` — only to whole 16-byte chunks (4 elements), which shrinks the footprint and gives up the alignment
+inline int padded_dims(int D, bool tight = false) { return tight ? (D + 3) / 4 * 4 : (D + 31) / 32 * 32; }
 // float4 registers per lane that hold a query of Dp elements spread over 16 lanes (template parameter QR
 // of the kernels); 0 = the query does not fit registers and is staged in LDS
 inline int query_regs(int Dp) {
@@ -786,6 +795,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
 template <int QR, bool HALF>
 __device__ __forceinline__ void load_node_query_t(QVec<QR>& qv, float4* qlds, const DevIndex& ix, uint32_t node, int lane) {
   const int rowlen = ix.Dp >> 2;
+  const int used = (ix.D + 3) >> 2;  // chunks that hold data (the last one zero padded)
   const uint64_t first = (uint64_t)node * (uint32_t)rowlen;
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
   if (QR > 0) {
@@ -793,17 +803,17 @@ __device__ __forceinline__ void load_node_query_t(QVec<QR>& qv, float4* qlds, co
 #pragma unroll
     for (int k = 0; k < (QR > 0 ? QR : 1); ++k) {
       const int c = sub + 16 * k;
-      const uint64_t at = first + (c < rowlen ? c : 0);  // unconditional load
+      const uint64_t at = first + (c < used ? c : 0);  // unconditional load
       const float4 t = HALF ? load_chunk_f16(ix.vectors, at) : load_chunk_f32(ix.vectors, at);
-      qv.q[k] = c < rowlen ? t : zero;
+      qv.q[k] = c < used ? t : zero;
     }
   } else {
-    const int chunks = (rowlen + 15) / 16 * 16;
+    const int chunks = (used + 15) / 16 * 16;
     wave_sync();
     for (int c = lane; c < chunks; c += 64) {
-      const uint64_t at = first + (c < rowlen ? c : 0);
+      const uint64_t at = first + (c < used ? c : 0);
       const float4 t = HALF ? load_chunk_f16(ix.vectors, at) : load_chunk_f32(ix.vectors, at);
-      qlds[c] = c < rowlen ? t : zero;
+      qlds[c] = c < used ? t : zero;
     }
     wave_sync();
   }
@@ -822,7 +832,7 @@ __device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, cons
 template <int DT, int QR>
 __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32_t* sid, const float* skey, int T, int m,
                                                 int nn_num, int save_remains, uint32_t* oid, float* okey, Scratch& s,
-                                                int lane) {
+                                                int lane, unsigned int* work = nullptr) {
   int head = 0;
   int tail = (m < T ? m : T) - 1;
   const int max_head = tail + 1;
@@ -840,6 +850,10 @@ __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32
     if (QR > 0 && j + 1 < T) load_node_query<QR>(cv_next, s.qlds, ix, sid[j + 1], lane);
     if (head >= nn_num && head > 0) {
       if (QR == 0) load_node_query<QR>(cv, s.qlds, ix, c, lane);
+      if (work && lane == 0) {  // (LDS: +2 pair tests, +3 candidate rows of this level's counters)
+        work[2] += (unsigned int)head;
+        work[3] += 1u;
+      }
       dist_list<DT, QR, false>(ix, cv, s.qlds, oid, head, s.dbuf, lane);
       wave_sync();
       bool mine = false;
@@ -885,6 +899,10 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
   float* okey = reinterpret_cast<float*>(smem + lp.out_key);
   s.tree = make_stage_tree(lane);
   bind_slot(s, a.pool, blockIdx.x);
+  // this wavefront's share of a.counters (LDS, so that counting costs the kernel no registers when it is off)
+  __shared__ unsigned int work[16];
+  if (lane < 16) work[lane] = 0u;
+  wave_sync();
 
   for (;;) {
     int b = 0;
@@ -914,6 +932,7 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
       for (int level = top_level; level >= 0; --level) {
         const int m_cap = level == 0 ? ix.max_m0 : ix.max_m;
         st.top_size = 0; st.cand_size = 0; st.n_acc = 0; st.lower = 0.f; st.maxkey = -INFINITY;
+        const int evals_before = st.n_dist, hops_before = st.n_hops;
         int T;
         if (sorted_set) {
           filter_reset(s, lane);
@@ -949,8 +968,15 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
           rank_sort(s.top, nullptr, T, sid, skey, lane);
           wave_sync();
         }
+        unsigned int* level_work = a.counters ? work + (level == 0 ? 0 : 5) : nullptr;
         const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, level == 0 ? a.own_cap0 : m_cap,
-                                                 level == 0 ? a.nn_num0 : a.nn_numU, a.save_remains, oid, okey, s, lane);
+                                                 level == 0 ? a.nn_num0 : a.nn_numU, a.save_remains, oid, okey, s, lane,
+                                                 level_work);
+        if (level_work && lane == 0) {
+          level_work[0] += (unsigned int)(st.n_dist - evals_before);
+          level_work[1] += (unsigned int)(st.n_hops - hops_before);
+          level_work[4] += 1u;
+        }
         if (QR == 0) load_node_query<QR>(qv, s.qlds, ix, x, lane);  // the LDS query copy was reused by the selection
         uint32_t* out_ids;
         float* out_keys;
@@ -974,8 +1000,14 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
         wave_sync();
       }
       if (lane == 0 && st.fail) *a.status = 1;
+      if (a.counters && lane == 0) {
+        work[5] += (unsigned int)st.n_dist_upper + (a.cur_max > lx ? 1u : 0u);  // the descent and its entry point
+        work[6] += (unsigned int)st.n_sweeps;
+      }
     }
   }
+  wave_sync();
+  if (a.counters && lane < 10 && work[lane] != 0u) atomicAdd(a.counters + lane, (unsigned long long)work[lane]);
 }
 
 __device__ __forceinline__ uint32_t* link_row_mut(const DevIndex& ix, uint32_t node, int level) {
@@ -1135,6 +1167,9 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
   uint32_t* oid = reinterpret_cast<uint32_t*>(smem + lp.out_id);
   float* okey = reinterpret_cast<float*>(smem + lp.out_key);
   const int n_dirty = *a.dirty_cnt;
+  __shared__ unsigned int work[16];
+  if (lane < 16) work[lane] = 0u;
+  wave_sync();
 
   for (int di = blockIdx.x; di < n_dirty; di += gridDim.x) {
     const unsigned long long entry = a.dirty[di];
@@ -1208,7 +1243,8 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
         rank_sort(cbuf, nullptr, T, sid, skey, lane);
         wave_sync();
         const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, m_cap, level == 0 ? a.nn_num0 : a.nn_numU,
-                                                 a.save_remains, oid, okey, s, lane);
+                                                 a.save_remains, oid, okey, s, lane,
+                                                 a.counters ? work + (level == 0 ? 0 : 5) : nullptr);
         for (int j = lane; j < m_cap; j += 64) {
           row[j] = j < deg ? oid[j] : kEmpty;
           drow[j] = j < deg ? okey[j] : 0.f;
@@ -1216,8 +1252,48 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       }
     }
     if (lane == 0) *cnt = 0;
+    if (a.counters && lane == 0) {
+      unsigned int* level_work = work + (level == 0 ? 0 : 5);
+      level_work[1] += 1u;
+      level_work[4] += n_new > 0 ? 1u : 0u;
+    }
     wave_sync();
   }
+  wave_sync();
+  if (a.counters && lane < 10 && work[lane] != 0u) atomicAdd(a.counters + lane, (unsigned long long)work[lane]);
+}
+
+// Measurement aid: nothing but the search's memory access pattern.  Every 16-lane group fetches pseudo-random
+// vector rows of the resident index, U rows per group in flight, each lane one 16-byte chunk per 64 elements,
+// exactly as the distance passes do; `dependent` makes each batch of loads wait for the one before, as a hop
+// waits for its rows.  Gives the rate at which this GPU's memory system delivers random rows of THIS index.
+template <int U>
+__global__ void __launch_bounds__(64) gather_probe_kernel(DevIndex ix, int batches, int dependent, float* sink) {
+  const int lane = threadIdx.x, g = lane >> 4, sub = lane & 15;
+  const uint32_t rowlen = (uint32_t)ix.Dp >> 2, used = ((uint32_t)ix.D + 3u) >> 2;
+  const int nk = (int)((used + 15u) >> 4);
+  uint32_t x = (uint32_t)(blockIdx.x * 4 + g) * 2654435761u + 12345u;
+  float acc = 0.f;
+  uint32_t chain = 0u;
+  for (int b = 0; b < batches; ++b) {
+    for (int k = 0; k < nk; ++k) {
+      float4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        uint32_t y = x + (uint32_t)u * 0x9E3779B9u;
+        y ^= y >> 15; y *= 0x2C1B3C6Du; y ^= y >> 12; y *= 0x297A2D39u; y ^= y >> 15;
+        const uint32_t id = (uint32_t)(((unsigned long long)y * (unsigned long long)ix.N) >> 32) + chain;
+        const uint32_t c = sub + 16u * (uint32_t)k;
+        const unsigned long long at = (unsigned long long)id * rowlen + (c < used ? c : 0u);
+        v[u] = ix.half ? load_chunk_f16(ix.vectors, at) : load_chunk_f32(ix.vectors, at);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+    }
+    x = x * 1664525u + 1013904223u;
+    if (dependent) chain = acc == 1234567.0f ? 1u : 0u;  // (never true: the next addresses just have to wait for this sum)
+  }
+  if (acc == 7654321.0f) sink[blockIdx.x] = acc;
 }
 
 // Upload helper for fp16 storage: N x D floats into rows of Dp halves (the padding was zeroed before).

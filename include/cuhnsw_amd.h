@@ -121,6 +121,20 @@ double cuhnsw_last_build_seconds(cuhnsw_engine* e);
  * (cpp/include/cuda_build_kernels.cuh:294-331).  Sets with hubs reach it: 0 on the 50- and 96-dimensional
  * benchmark configurations, about 12 600 of 25 million links on the 1 M x 128 integer-valued one. */
 int cuhnsw_last_build_dropped_links(cuhnsw_engine* e);
+/* Measurement aid (no counterpart in the reference): the search's memory access pattern alone.  waves_per_cu
+ * wavefronts per CU fetch pseudo-random vector rows of the resident index, 16 lanes per row, rows_in_flight
+ * (4, 8 or 16) rows per wavefront at a time; dependent != 0 makes every batch of loads wait for the previous
+ * one, as a hop of the search waits for its rows.  rows receives the number of rows fetched, ms the kernel
+ * time (best of three): rows x 4 x num_dims / ms is the rate at which this GPU delivers random rows of this
+ * index, the ceiling the search's gather phase is measured against. */
+int cuhnsw_debug_gather_probe(cuhnsw_engine* e, int waves_per_cu, int rows_in_flight, int dependent, double* rows,
+                              float* ms);
+/* Work of the last cuhnsw_build_graph, counted on the device when tunable "build_counters" = 1 was set before it
+ * (all zero otherwise); the reference counts its visited nodes per level the same way
+ * (cpp/src/cuhnsw_build.cu:191-195).  out[0..4] level 0, out[5..9] upper levels: distance evaluations of the
+ * searches and descents, link rows read, pair tests of the selection heuristic, candidates the heuristic loaded
+ * to test them, link rows written.  n must be at least 10. */
+int cuhnsw_last_build_counters(cuhnsw_engine* e, unsigned long long* out, int n);
 /* Debugging aid: the key (ordering distance) the build stored with every level-0 link, row-major
  * [num_data x max_m0] in list order, as the reference keeps them in its `distances` array
  * (cpp/include/cuda_build_kernels.cuh:270-278).  Needs tunable "keep_link_keys" = 1 before build_graph. */
@@ -156,6 +170,7 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   it leaves and the host answers the remaining queries afterwards (-1 = no bound in
  *                   polls: it leaves when the first pass has not started within 2 ms or stalls for
  *                   100 ms, and the engine then runs the passes one after the other from then on)
+ *   "build_counters" 1 = count the work of the next builds on the device (cuhnsw_last_build_counters)
  *   "keep_link_keys" 1 = keep the keys stored with the level-0 links after build_graph for
  *                   cuhnsw_debug_link_keys0
  *   "lean_literal"  visited set of the literal-queue pass: 0 = exact bitmap in HBM (one bit per point and
@@ -164,6 +179,9 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)
+ *   "tight_rows"    1 = vector rows are padded to whole 16-byte chunks only instead of 128-byte lines (D = 50:
+ *                   208 instead of 256 bytes per row).  Smaller footprint, rows no longer line-aligned; same
+ *                   results.  Has to be set before set_data / load_index (returns -2 afterwards).  Default 0.
  *   "fp16_storage"  1 = the vectors are kept in device memory as fp16 (the reference's switched-off
  *                   HALF_PRECISION idea, cpp/include/types.hpp:9-28).  The index then IS an index over
  *                   the vectors rounded to fp16 (nearest even; magnitudes beyond 65504 become

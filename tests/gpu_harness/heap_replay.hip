@@ -48,12 +48,12 @@ extern "C" int heap_replay(const float* keys, int n_ops, int minq, int lds_cap, 
   int *d_sizes = nullptr, *d_popped = nullptr;
   const int n_dumps = n_ops / dump_every;
   if (hipMalloc(&d_keys, sizeof(float) * n_ops) != hipSuccess) return 1;
-  hipMalloc(&d_glob, sizeof(HeapEnt) * cap);
-  hipMalloc(&d_dumps, sizeof(HeapEnt) * (size_t)cap * (n_dumps + 1));
-  hipMalloc(&d_sizes, sizeof(int) * (n_dumps + 1));
-  hipMalloc(&d_popped, sizeof(int) * n_ops);
-  hipMemcpy(d_keys, keys, sizeof(float) * n_ops, hipMemcpyHostToDevice);
-  hipMemset(d_dumps, 0, sizeof(HeapEnt) * (size_t)cap * (n_dumps + 1));
+  (void)hipMalloc(&d_glob, sizeof(HeapEnt) * cap);
+  (void)hipMalloc(&d_dumps, sizeof(HeapEnt) * (size_t)cap * (n_dumps + 1));
+  (void)hipMalloc(&d_sizes, sizeof(int) * (n_dumps + 1));
+  (void)hipMalloc(&d_popped, sizeof(int) * n_ops);
+  (void)hipMemcpy(d_keys, keys, sizeof(float) * n_ops, hipMemcpyHostToDevice);
+  (void)hipMemset(d_dumps, 0, sizeof(HeapEnt) * (size_t)cap * (n_dumps + 1));
   if (minq)
     hipLaunchKernelGGL(replay_kernel<true>, dim3(1), dim3(64), (size_t)lds_cap * 8, 0, d_keys, n_ops, lds_cap, d_glob,
                        d_dumps, cap, dump_every, d_sizes, d_popped);
@@ -62,13 +62,13 @@ extern "C" int heap_replay(const float* keys, int n_ops, int minq, int lds_cap, 
                        d_dumps, cap, dump_every, d_sizes, d_popped);
   int rc = hipDeviceSynchronize() == hipSuccess ? 0 : 2;
   std::vector<HeapEnt> host((size_t)cap * n_dumps);
-  hipMemcpy(host.data(), d_dumps, sizeof(HeapEnt) * host.size(), hipMemcpyDeviceToHost);
+  (void)hipMemcpy(host.data(), d_dumps, sizeof(HeapEnt) * host.size(), hipMemcpyDeviceToHost);
   for (size_t i = 0; i < host.size(); ++i) {
     dump_keys[i] = host[i].key;
     dump_ids[i] = host[i].id;
   }
-  hipMemcpy(sizes, d_sizes, sizeof(int) * n_dumps, hipMemcpyDeviceToHost);
-  hipMemcpy(popped, d_popped, sizeof(int) * n_ops, hipMemcpyDeviceToHost);
-  hipFree(d_keys); hipFree(d_glob); hipFree(d_dumps); hipFree(d_sizes); hipFree(d_popped);
+  (void)hipMemcpy(sizes, d_sizes, sizeof(int) * n_dumps, hipMemcpyDeviceToHost);
+  (void)hipMemcpy(popped, d_popped, sizeof(int) * n_ops, hipMemcpyDeviceToHost);
+  (void)hipFree(d_keys); (void)hipFree(d_glob); (void)hipFree(d_dumps); (void)hipFree(d_sizes); (void)hipFree(d_popped);
   return rc;
 }

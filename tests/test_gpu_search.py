@@ -145,6 +145,29 @@ def test_two_queries_per_wavefront_equal_one_per_wavefront(oracle, tmp_path, nam
   e.set_tunable("pair_path", 1)
 
 
+def test_tight_rows_layout_and_gather_probe(oracle, tmp_path):
+  """Vector rows padded to 16-byte chunks only (tunable tight_rows; rows then start off the 128-byte lines):
+  same answers as the oracle, for a dimension with a partial last chunk too.  And the memory-pattern probe
+  runs on the resident vectors and reports a sane rate."""
+  for d, dist in ((50, "dot"), (7, "l2"), (100, "l2")):
+    n = 3000
+    x = gauss_mixture(n, d, seed=41, normalise=(dist == "dot"))
+    q = gauss_mixture(100, d, seed=42, normalise=(dist == "dot"))
+    mult = 1 / np.log(8)
+    ix = oracle.OracleIndex(dist).build(x, _levels(n, mult, 43), 8, 16, 60, mult)
+    p = str(tmp_path / "tight.idx")
+    ix.save(p)
+    e = _engine(tmp_path, dist_type=dist, max_m=8, max_m0=16)
+    e.set_tunable("tight_rows", 1)
+    e.load_index(p)
+    with pytest.raises(RuntimeError, match="before set_data"):
+      e.set_tunable("tight_rows", 0)
+    _check_parity(oracle, ix, e, q, 10, 100)
+    _check_parity(oracle, ix, e, q, 10, 300)
+    rows, ms = e.gather_probe(8, 4, True)
+    assert rows > 0 and rows % (8 * 4 * 2048) == 0 and 0.0 < ms < 1000.0
+
+
 def test_labels_from_file_are_returned(oracle, tmp_path):
   n, d = 3000, 20
   x = gauss_mixture(n, d, seed=4)
