@@ -121,8 +121,8 @@ def main():
                   help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   ap.add_argument("--fast-path", type=int, default=1, choices=[0, 1, 2],
                   help="0 = literal priority queues only, 1 = default, 2 = sorted-set first pass whatever the batch size")
-  ap.add_argument("--pair-path", type=int, default=1, choices=[0, 1],
-                  help="0 = never two queries per wavefront in the first pass")
+  ap.add_argument("--pair-path", type=int, default=1, choices=[0, 1, 2],
+                  help="0 = never two queries per wavefront in the first pass, 2 = wherever the shapes allow it")
   ap.add_argument("--no-large", action="store_true", help="skip the extra 4x batch (profiling runs)")
   ap.add_argument("--profile", action="store_true",
                   help="profiling run: only searches of the default path are launched (no literal-only counting pass, "
@@ -314,7 +314,7 @@ def main():
                     "queries_repeated_with_literal_queues": int(repeats)},
       "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                    "frac": achieved / 8000.0, "traffic": traffic,
-                   "kernel": ("search_pair_kernel" if (args.pair_path and ef <= 128 and d <= 128) else "search_fast_kernel") +
+                   "kernel": ("search_pair_kernel" if (args.pair_path and d <= 128 and (ef <= 64 or (ef <= 128 and nq >= 14336))) else "search_fast_kernel") +
                              " with search_kernel beside it (one search of the batch)"
                              if args.fast_path else "search_kernel (literal priority queues only)",
                    "algorithmic_bytes_per_launch": gather_bytes},

@@ -474,7 +474,14 @@ class Engine {
       constexpr bool kPairShape = (QR == 1 || QR == 2) && NS == 2;
       constexpr int N2 = kPairShape ? 2 * NS : 2;
       auto pair_kernel = search_pair_kernel<DT, (kPairShape ? QR : 1), N2>;
-      const bool pair = kPairShape && pair_path != 0 && !a.reverse && host.S0 <= 32 && host.SU <= 32 && a.nq > 1;
+      // (measured: at ef_search up to 64 the pair kernel is the faster one whatever the batch; between 65 and 128
+      // it wins once the batch is several rounds of wavefronts — 1.18 M x 50, 40 000 queries, ef 128: 5.5 against
+      // 6.5 ms; 10 M x 96, 100 000 queries: 20.0 against 21.3 ms — and loses where the whole batch is resident at
+      // once and a query's own latency is what counts — 1 M x 128, 10 000 queries, ef 128: 2.95 against 2.68 ms;
+      // pair_path = 2 forces it)
+      const int single_slots = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits).total);
+      const bool pair = kPairShape && pair_path != 0 && !a.reverse && host.S0 <= 32 && host.SU <= 32 && a.nq > 1 &&
+                        (pair_path > 1 || a.ef <= 64 || a.nq >= 2 * single_slots);
       auto fast_lds = [&](int bits) -> size_t {
         return pair ? plan_pair_lds(a.lcap, bits).total : plan_fast_lds(QR, ix.Dp, a.lcap, bits).total;
       };

@@ -158,9 +158,10 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   batch exceeds one round of resident wavefronts, literal queues for the queries
  *                   that met equal distances (default); 2 = first pass whatever the batch size
  *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
- *   "pair_path"     1 = the first pass runs two queries per wavefront (32 lanes each) where ef_search is at
- *                   most 128, the vectors have at most 128 dimensions and max_m, max_m0 at most 32
- *                   (default); 0 = always one query per wavefront.  Same results either way.
+ *   "pair_path"     1 = the first pass runs two queries per wavefront (32 lanes each) where that is the faster
+ *                   shape: ef_search up to 64, or up to 128 with a batch of several rounds of wavefronts; vectors
+ *                   of at most 128 dimensions, max_m and max_m0 at most 32 (default); 2 = wherever the shapes
+ *                   allow it (ef_search up to 128); 0 = always one query per wavefront.  Same results either way.
  *   "first_pass_waves" wavefronts per CU of the first pass (0 = as many as fit, the default)
  *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
  *                   (default), 0 = after it
