@@ -5,6 +5,7 @@ reference's examples/example1.py, which needs downloads, h5py and hnswlib).
   python examples/example_synthetic.py run_gpu_training  --workload C1 --index /tmp/c1.idx
   python examples/example_synthetic.py run_gpu_inference --workload C1 --index /tmp/c1.idx --topk 10 --ef-search 300
   python examples/example_synthetic.py run_experiments   --workload C1
+  python examples/example_synthetic.py run_knob_sweep    --workload C2 --ef-list 30 50 300
 
 Recall is measured against exact neighbours computed on the GPU with a plain matmul.
 If the `hnswlib` package is importable, `run_cpu_inference` searches the same index file
@@ -104,9 +105,38 @@ def run_experiments(args):
       print("| %d | %.3f | %d | %.0f | %.4f |" % (efc, build_s, ef, queries.shape[0] / el, recall(nns, truth)))
 
 
+def run_knob_sweep(args):
+  """Build-side knobs the reference took over from n2 (README.md:97-98,104 of the reference): heuristic_coef
+  (share of every link row filled with the nearest candidates untested), save_remains (pruned candidates fill
+  the row) and reverse_cand (the farthest waiting candidate is expanded first during construction): build time
+  and recall at several ef_search, all searched the same (plain) way."""
+  data, queries, spec = datasets.make(args.workload, n=args.n)
+  truth = exact_neighbours(data, queries, args.topk, spec["opt"]["dist_type"])
+  efs = args.ef_list or [30, 50, 300]
+  print("| heuristic_coef | save_remains | reverse_cand | build s | " + " | ".join("recall@%d ef %d" % (args.topk, e) for e in efs) + " |")
+  print("|---|---|---|---|" + "---|" * len(efs))
+  for coef, remains, reverse in ((0.0, False, False), (0.25, False, False), (0.5, False, False), (0.0, True, False),
+                                 (0.25, True, False), (0.0, False, True), (0.25, False, True)):
+    h = CuHNSW(dict(options(spec), heuristic_coef=coef, save_remains=remains, reverse_cand=reverse))
+    h.set_data(data)
+    h.build()
+    build_s = h.obj.last_build_seconds()
+    path = args.index + ".sweep"
+    h.save_index(path)
+    plain = CuHNSW(options(spec))            # search without reverse_cand, whatever the build used
+    plain.load_index(path)
+    os.remove(path)
+    cells = []
+    for ef in efs:
+      nns, _, _ = plain.search_knn(queries, args.topk, ef)
+      cells.append("%.4f" % recall(nns, truth))
+    print("| %.2f | %s | %s | %.3f | %s |" % (coef, remains, reverse, build_s, " | ".join(cells)), flush=True)
+
+
 def main():
   ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-  ap.add_argument("command", choices=["run_gpu_training", "run_gpu_inference", "run_cpu_inference", "run_experiments"])
+  ap.add_argument("command", choices=["run_gpu_training", "run_gpu_inference", "run_cpu_inference", "run_experiments",
+                                      "run_knob_sweep"])
   ap.add_argument("--workload", default="C1", choices=sorted(datasets.CONFIGS))
   ap.add_argument("--n", type=int, default=None, help="shrink the data set")
   ap.add_argument("--index", default="/tmp/cuhnsw_amd_example.idx")
