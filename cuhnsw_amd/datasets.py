@@ -29,6 +29,12 @@ CONFIGS = {
                nq=100_000, topk=100, ef=[64, 128, 256, 512],
                opt=dict(dist_type="dot", max_m=16, max_m0=32,
                         ef_construction=150)),
+    # the run the reference's README times (examples/example1.py:206-226 there): the 1 183 514 x 50 angular
+    # index, ONE batch of 1 000 000 random unit vectors as queries, topk 100, ef_search 300
+    "R1": dict(cfg=2, n=1_183_514, d=50, centres=1000, law="gauss_nrz", query_law="unit_normal",
+               nq=1_000_000, topk=100, ef=[300],
+               opt=dict(dist_type="dot", max_m=12, max_m0=24,
+                        ef_construction=110)),
 }
 
 
@@ -69,8 +75,12 @@ def make(name, n=None, nq=None):
   rng = np.random.default_rng(1000 + spec["cfg"])
   centres = _centres(rng, spec["law"], spec["centres"], spec["d"])
   data = _draw(rng, centres, spec["law"], n)
-  queries = _draw(np.random.default_rng(2000 + spec["cfg"]), centres,
-                  spec["law"], nq)
+  qrng = np.random.default_rng(2000 + spec["cfg"])
+  if spec.get("query_law") == "unit_normal":
+    queries = qrng.standard_normal((nq, spec["d"])).astype(np.float32)
+    queries /= np.linalg.norm(queries, axis=1, keepdims=True)
+  else:
+    queries = _draw(qrng, centres, spec["law"], nq)
   spec["n"], spec["nq"] = n, nq
   return data, queries, spec
 

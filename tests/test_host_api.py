@@ -130,3 +130,9 @@ def test_datasets_are_seeded_and_shaped():
   g, _, _ = datasets.make("C4", n=100, nq=10)
   assert g.shape == (100, 960) and g.min() >= 0 and g.max() <= 1
   assert spec["opt"]["level_mult"] == pytest.approx(1 / np.log(24))
+  # the reference README's run shape: the C2 data (same seed), queries uniform on the unit sphere
+  r, qr, rs = datasets.make("R1", n=500, nq=40)
+  c2, _, _ = datasets.make("C2", n=500, nq=1)
+  assert (r == c2).all() and qr.shape == (40, 50) and rs["topk"] == 100
+  np.testing.assert_allclose(np.linalg.norm(qr, axis=1), 1.0, rtol=1e-5)
+  assert abs(float(qr.mean())) < 0.05
