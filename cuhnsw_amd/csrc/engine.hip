@@ -117,7 +117,7 @@ class Engine {
   double last_build_seconds = 0.0;
 
   // tunables
-  int build_batch = 16384;
+  int build_batch = 0;     // nodes inserted per batch at most; 0 = by the size of the graph (batch_at)
   int search_slots = 0;
   int cand_lds_override = 0;
   int hnswlib_dist = 0;
@@ -727,7 +727,7 @@ class Engine {
   void build_levels() {
     const int N = host.N;
     const int cap_in = 32;
-    const int bmax = std::max(1, build_batch);
+    const int bmax = build_batch > 0 ? build_batch : std::min(std::max(N, 1), 65536);
     const int m_max = std::max(host.max_m, host.max_m0);
     const size_t up_rows = std::max<size_t>((size_t)host.upper_rows, 1);
     DevBuf<float> d_dists0, d_distsU, d_sel0_keys, d_selU_keys;
@@ -803,12 +803,21 @@ class Engine {
 
     // Nodes go in by ascending id, as hnswlib inserts them.  The graph a batch sees is the
     // one of all earlier batches: its entry point is the first node that reached the highest
-    // level so far.  Batches grow with the graph (a quarter of what is already in) up to
-    // build_batch, so that early nodes, which wire the long-range links, see each other.
+    // level so far.  Batches grow with the graph — a quarter of what is already in, up to 16 384 nodes, so
+    // that early nodes, which wire the long-range links, see each other; beyond half a million nodes a
+    // thirty-second of the graph, up to 65 536 — because the nodes of a batch do not see each other, and a
+    // launch of several rounds of wavefronts loses less to its last, partly filled round (1.18 M x 50: 0.224 s
+    // with batches of 16 384 throughout, 0.171 s with 65 536, recall unchanged; 1 M x 960: recall@10 at
+    // ef_search 300 0.9831 / 0.9812, at 50 0.836 / 0.829, which is why the share of new nodes stays small).
+    // build_batch > 0 replaces the two caps by one.
+    auto batch_at = [&](int in) {
+      if (build_batch > 0) return std::max(1, std::min(build_batch, in / 4));
+      return std::max(1, std::min(in / 4, std::max(16384, std::min(65536, in / 32))));
+    };
     int cur_ep = 0, cur_max = -1;
     int pos = 0;
     while (pos < N) {
-      int b = std::max(1, std::min(bmax, pos / 4));
+      int b = batch_at(pos);
       b = std::min(b, N - pos);
       a.begin = pos;
       a.count = b;

@@ -145,7 +145,8 @@ int cuhnsw_debug_link_keys0(cuhnsw_engine* e, float* out, long long capacity);
  * because its kernel does not reproduce hnswlib's tie order) */
 int cuhnsw_last_search_repeats(cuhnsw_engine* e);
 /* tuning knobs that are not part of the reference's option table:
- *   "build_batch"   largest number of nodes inserted per batch (default 16384)
+ *   "build_batch"   largest number of nodes inserted per batch (default 0 = by the size of the graph: a quarter
+ *                   of the nodes already in, at most 16384; beyond 524288 nodes a thirty-second, at most 65536)
  *   "search_slots"  resident wavefronts used by search (0 = automatic)
  *   "cand_lds"      candidate-queue entries kept in LDS (0 = automatic)
  *   "hnswlib_dist"  1 = return hnswlib distances (1-dot) instead of -dot
