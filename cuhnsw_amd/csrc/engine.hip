@@ -117,6 +117,7 @@ class Engine {
   double last_build_seconds = 0.0;
 
   // tunables
+  int level_first = 1;     // build: a batch hands out its nodes with upper levels first
   int build_batch = 0;     // nodes inserted per batch at most; 0 = by the size of the graph (batch_at)
   int search_slots = 0;
   int cand_lds_override = 0;
@@ -814,6 +815,26 @@ class Engine {
       if (build_batch > 0) return std::max(1, std::min(build_batch, in / 4));
       return std::max(1, std::min(in / 4, std::max(16384, std::min(65536, in / 32))));
     };
+    // within a batch the nodes with upper levels are handed out first (highest level first, then by id)
+    DevBuf<int> d_order;
+    {
+      std::vector<int> order((size_t)N);
+      for (int p0 = 0; p0 < N;) {
+        const int b = std::min(batch_at(p0), N - p0);
+        int* o = order.data() + p0;
+        int n_up = 0;
+        for (int i = 0; i < b; ++i)
+          if (host.levels[p0 + i] > 0) o[n_up++] = i;
+        std::stable_sort(o, o + n_up, [&](int x, int y) { return host.levels[p0 + x] > host.levels[p0 + y]; });
+        for (int i = 0, w = n_up; i < b; ++i)
+          if (host.levels[p0 + i] <= 0) o[w++] = i;
+        p0 += b;
+      }
+      d_order.reserve((size_t)N);
+      HIP_CHECK(hipMemcpyAsync(d_order.p, order.data(), (size_t)N * sizeof(int), hipMemcpyHostToDevice, stream));
+      HIP_CHECK(hipStreamSynchronize(stream));
+    }
+    a.order = level_first ? d_order.p : nullptr;
     int cur_ep = 0, cur_max = -1;
     int pos = 0;
     while (pos < N) {
@@ -1071,6 +1092,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   if (!e || !name) return -1;
   std::string n(name);
   if (n == "build_batch") e->impl.build_batch = (int)value;
+  else if (n == "level_first") e->impl.level_first = (int)value;
   else if (n == "search_slots") e->impl.search_slots = (int)value;
   else if (n == "cand_lds") e->impl.cand_lds_override = (int)value;
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;

@@ -75,6 +75,9 @@ struct SearchArgs {
 
 struct BuildArgs {
   int begin, count;        // batch = nodes begin .. begin+count-1
+  const int* order;        // N entries or null: the i-th node a batch hands out is begin + order[begin + i] (the
+                           // nodes with upper levels first: they take several searches, and a launch ends when
+                           // its last node does)
   int cur_ep, cur_max;     // entry point and top level of the graph before this batch (cur_max < 0: empty)
   int efc, nn_num0, nn_numU, save_remains;
   int reverse;   // expand the farthest waiting candidate (reverse_cand)
@@ -906,7 +909,10 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
 
   for (;;) {
     int b = 0;
-    if (lane == 0) b = atomicAdd(a.counter, 1);
+    if (lane == 0) {
+      b = atomicAdd(a.counter, 1);
+      if (b < a.count && a.order) b = a.order[a.begin + b];
+    }
     b = __builtin_amdgcn_readfirstlane(b);
     if (b >= a.count) break;
     const uint32_t x = (uint32_t)(a.begin + b);

@@ -147,6 +147,8 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
 /* tuning knobs that are not part of the reference's option table:
  *   "build_batch"   largest number of nodes inserted per batch (default 0 = by the size of the graph: a quarter
  *                   of the nodes already in, at most 16384; beyond 524288 nodes a thirty-second, at most 65536)
+ *   "level_first"   1 (default) = a build batch hands out its nodes with upper levels first (they take several
+ *                   searches each, and a launch ends when its last node does); 0 = by id.  Same graph either way.
  *   "search_slots"  resident wavefronts used by search (0 = automatic)
  *   "cand_lds"      candidate-queue entries kept in LDS (0 = automatic)
  *   "hnswlib_dist"  1 = return hnswlib distances (1-dot) instead of -dot
