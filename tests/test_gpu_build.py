@@ -160,6 +160,31 @@ def test_build_is_deterministic(tmp_path):
   assert files[0] == files[1]
 
 
+def test_hand_out_order_and_batch_cap_tunables(oracle, tmp_path):
+  """Which node of a batch a wavefront takes next (upper-level nodes first, or by id) cannot change the graph: the
+  batch reads the graph of the earlier batches only.  The batch cap can: a single cap of 2 000 nodes is another
+  (valid) schedule."""
+  from cuhnsw_amd import capi
+  x = gauss_mixture(30000, 32, centres=150, seed=71)
+  levels = _levels(30000, 0.45, 72)
+  path, _ = write_options(tmp_path, dist_type="dot", max_m=8, max_m0=16, ef_construction=60)
+  files = {}
+  for tag, tunables in (("first", {"level_first": 1}), ("by_id", {"level_first": 0}), ("cap", {"build_batch": 2000})):
+    e = capi.Engine()
+    assert e.init(path) == 0
+    for k, v in tunables.items():
+      e.set_tunable(k, v)
+    e.set_data(x)
+    e.set_random_levels(levels)
+    e.build_graph()
+    p = str(tmp_path / (tag + ".idx"))
+    e.save_index(p)
+    files[tag] = open(p, "rb").read()
+    assert oracle.OracleIndex("dot").load(p).validate() == 0
+  assert files["first"] == files["by_id"]
+  assert files["cap"] != files["first"]
+
+
 def test_option_variants_keep_invariants(oracle, tmp_path):
   x = gauss_mixture(5000, 16, seed=41)
   levels = _levels(5000, 0.5, 42)
