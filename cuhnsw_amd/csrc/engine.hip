@@ -129,6 +129,7 @@ class Engine {
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   int first_pass_waves = 0;  // wavefronts per CU of the first pass (0 = as many as fit)
   int pair_path = 1;       // first pass with two queries per wavefront where the shapes allow it (0: one per wavefront)
+  int query_order = 1;     // first pass of two or more rounds of wavefronts: longest queries first (0: caller's order)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
   bool storage_half = false;  // vectors live in HBM as fp16 (set before set_data / load_index)
@@ -160,6 +161,9 @@ class Engine {
   DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count, [32] queries given up by the
                       // sorted-set pass, [64] queries it has finished with, [96] work counter of a concurrent literal pass
   DevBuf<int> d_redo;  // their indices
+  DevBuf<uint4> d_entry;      // longest queries first: level-0 entry of every query of the batch,
+  DevBuf<int> d_order_hist;   // bucket counters,
+  DevBuf<int> d_order;        // and the order the first pass takes the queries in
   // staging for the host-pointer search entry point
   DevBuf<float> d_q, d_dist;
   DevBuf<int> d_nns, d_found;
@@ -433,6 +437,9 @@ class Engine {
     a.start_ticks = 2 * wall_clock_khz;
     a.stall_ticks = 100 * wall_clock_khz;
     a.nq_dev = nullptr;
+    a.entry = nullptr;
+    a.order_hist = nullptr;
+    a.order = nullptr;
     last_repeats = 0;
     if (use_static) {
       launch_search_static<DT, QR, NS>(ix, a, ms);
@@ -517,16 +524,49 @@ class Engine {
       slots = std::max(1, std::min(slots, pair ? (a.nq + 1) / 2 : a.nq));
       HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 128 * sizeof(int), stream));
       HIP_CHECK(hipMemsetAsync(d_redo.p, 0xFF, (size_t)a.nq * sizeof(int), stream));
+      // (every allocation before the literal pass is launched: growing a buffer frees the old one, and
+      // hipFree waits for the device, on which that pass would be waiting for the first pass to start)
+      // (from two rounds of wavefronts on — 1.18 M x 50, 40 000 queries: 8.25 -> 7.41 ms; at 1.45 rounds, 10 000
+      // queries, the first pass alone gains, 2.46-2.76 -> 2.14 ms, but its heavy queries then hand over late and the
+      // batch ends no earlier, 3.2 against 3.0-3.1 ms; query_order = 2 puts any batch of more than one round in order)
+      const bool in_order = query_order && !pair && (query_order > 1 ? a.nq > slots : a.nq >= 2 * slots);
+      if (in_order) {
+        d_entry.reserve((size_t)a.nq);
+        d_order.reserve((size_t)a.nq);
+        d_order_hist.reserve((size_t)kOrderBuckets);
+      }
       if (side) {
         SearchArgs b = a;
         b.live = 1;
         b.counter = d_ctl.p + 96;
         b.pool = pool;
+        // (the first pass starts after the batch's descents when its queries are put in order: 0.1 ms per
+        // 10 000 queries of the 1.18 M x 50 set; allow ten times that on top of the usual 2 ms)
+        b.start_ticks += (long long)wall_clock_khz * (a.nq / 10000 + 1);
         HIP_CHECK(hipEventRecord(ev_side0, stream));
         HIP_CHECK(hipStreamWaitEvent(stream2, ev_side0, 0));
         hipLaunchKernelGGL(kernel, dim3(side_slots), dim3(64), lp.total, stream2, ix, b);
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipEventRecord(ev_side1, stream2));
+      }
+      // more than one round of wavefronts: the batch's descents first, then its queries longest first.  (The
+      // literal pass has been launched by now: launched after the first pass it would find no room until the
+      // first of that pass's wavefronts leave, a third of the way through the batch.)
+      if (in_order) {
+        a.entry = d_entry.p;
+        a.order = d_order.p;
+        a.order_hist = d_order_hist.p;
+        HIP_CHECK(hipMemsetAsync(d_order_hist.p, 0, (size_t)kOrderBuckets * sizeof(int), stream));
+        auto k_entry = entry_kernel<DT, QR>;
+        const size_t entry_lds = plan_fast_lds(QR, ix.Dp, a.lcap, 0).total;
+        const int entry_grid = std::max(1, std::min(a.nq, resident_slots(k_entry, entry_lds)));
+        hipLaunchKernelGGL(k_entry, dim3(entry_grid), dim3(64), entry_lds, stream, ix, a);
+        HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(order_prefix_kernel, dim3(1), dim3(1024), 0, stream, d_order_hist.p);
+        HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(order_scatter_kernel, dim3((unsigned)((a.nq + 255) / 256)), dim3(256), 0, stream, d_entry.p,
+                           a.nq, d_order_hist.p, d_order.p);
+        HIP_CHECK(hipGetLastError());
       }
       if (pair) hipLaunchKernelGGL(pair_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
       else hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
@@ -1102,6 +1142,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "lean_literal") e->impl.lean_literal = (int)value;
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
   else if (n == "pair_path") e->impl.pair_path = (int)value;
+  else if (n == "query_order") e->impl.query_order = (int)value;
   else if (n == "first_pass_waves") e->impl.first_pass_waves = (int)value;
   else if (n == "concurrent_literal") e->impl.concurrent_literal = value != 0.0;
   else if (n == "literal_spin_limit") e->impl.spin_limit_override = (int)value;

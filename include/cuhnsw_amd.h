@@ -161,6 +161,10 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   batch exceeds one round of resident wavefronts, literal queues for the queries
  *                   that met equal distances (default); 2 = first pass whatever the batch size
  *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
+ *   "query_order"   1 (default) = a search batch of two or more rounds of wavefronts does its upper-level descents
+ *                   first and takes its queries by descending distance of their level-0 entry point (the longest
+ *                   searches first: a launch ends when its last query does); 2 = from more than one round on;
+ *                   0 = in the caller's order.  Same answers and counters either way.
  *   "pair_path"     1 = the first pass runs two queries per wavefront (32 lanes each) where that is the faster
  *                   shape: ef_search up to 64, or up to 128 with a batch of several rounds of wavefronts; vectors
  *                   of at most 128 dimensions, max_m and max_m0 at most 32 (default); 2 = wherever the shapes

@@ -145,6 +145,33 @@ def test_two_queries_per_wavefront_equal_one_per_wavefront(oracle, tmp_path, nam
   e.set_tunable("pair_path", 1)
 
 
+@pytest.mark.parametrize("kind,d,dist", [("gauss", 50, "dot"), ("int", 24, "l2")], ids=["dot50", "l2_int_ties"])
+def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, kind, d, dist):
+  """A batch of several rounds of wavefronts does its upper-level descents first and takes its queries by
+  descending entry distance.  Answers, found counts and every counter (the descent's evaluations and sweeps come
+  from the separate kernel) are those of the caller's order, and the oracle's."""
+  n, nq, k, ef = 8000, 9000, 10, 150
+  x = _data(kind, n, d, 11)
+  q = _data(kind, nq, d, 12)
+  ix = oracle.OracleIndex(dist).build(x, _levels(n, 0.4, 13), 8, 16, 60, 0.4)
+  p = str(tmp_path / "i.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type=dist, max_m=8, max_m0=16)
+  e.load_index(p)
+  e.set_tunable("pair_path", 0)
+  got = {}
+  for order in (2, 0):          # 2: in order whenever the batch is more than one round of wavefronts
+    e.set_tunable("query_order", order)
+    got[order] = _device_search(e, q, k, ef)
+  for a, b in zip(got[2], got[0]):
+    assert (a == b).all()
+  o_ids, o_d, o_f, o_cnt = ix.search(q[:1500], k, ef, counters=True)
+  g_ids, g_d, g_f, stats = got[2]
+  assert (g_f[:1500] == o_f).all() and (g_ids[:1500] == o_ids).all() and (g_d[:1500] == o_d).all()
+  assert (stats[:1500, 1:] == o_cnt[:, 1:4]).all()
+  e.set_tunable("query_order", 1)
+
+
 def test_tight_rows_layout_and_gather_probe(oracle, tmp_path):
   """Vector rows padded to 16-byte chunks only (tunable tight_rows; rows then start off the 128-byte lines):
   same answers as the oracle, for a dimension with a partial last chunk too.  And the memory-pattern probe
