@@ -529,7 +529,8 @@ class Engine {
       // (from two rounds of wavefronts on — 1.18 M x 50, 40 000 queries: 8.25 -> 7.41 ms; at 1.45 rounds, 10 000
       // queries, the first pass alone gains, 2.46-2.76 -> 2.14 ms, but its heavy queries then hand over late and the
       // batch ends no earlier, 3.2 against 3.0-3.1 ms; query_order = 2 puts any batch of more than one round in order)
-      const bool in_order = query_order && !pair && (query_order > 1 ? a.nq > slots : a.nq >= 2 * slots);
+      const long long resident = pair ? 2LL * slots : slots;  // queries at work at a time
+      const bool in_order = query_order && (query_order > 1 ? a.nq > resident : a.nq >= 2 * resident);
       if (in_order) {
         d_entry.reserve((size_t)a.nq);
         d_order.reserve((size_t)a.nq);

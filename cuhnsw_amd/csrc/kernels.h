@@ -406,7 +406,10 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
     // ---- a half without a query takes the next one ------------------------------------------------------
     if (wave_any(phase == PP_NEED)) {
       int got = 0;
-      if (phase == PP_NEED && hl == 0) got = atomicAdd(a.counter, 1);
+      if (phase == PP_NEED && hl == 0) {
+        got = atomicAdd(a.counter, 1);
+        if (got < a.nq && a.order) got = a.order[got];  // longest queries first
+      }
       got = half_read(got, 0, lane);
       if (phase == PP_NEED) {
         if (got >= a.nq) {
@@ -431,6 +434,19 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
           n_dist = 0; n_hops = 0; n_dist_upper = 0; n_sweeps = 0;
           cur = ix.enterpoint;
           phase = PP_ENTRY;
+          if (a.entry) {
+            // the descent through the upper levels has been done for the whole batch: straight to level 0,
+            // with a fresh sorted set and visited filter
+            const uint4 en = a.entry[qi];
+            cur = en.x;
+            n_dist_upper = (int)en.z;
+            n_sweeps = (int)en.w;
+            phase = PP_SEED;
+            pf_init<N>(fr, ef, hl);
+            uint4* c4 = reinterpret_cast<uint4*>(sets);
+            const int n4 = (1 << a.fc_bits) >> 2;
+            for (int i = hl; i < n4; i += 32) c4[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+          }
         }
       }
     }

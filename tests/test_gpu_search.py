@@ -150,7 +150,7 @@ def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, k
   """A batch of several rounds of wavefronts does its upper-level descents first and takes its queries by
   descending entry distance.  Answers, found counts and every counter (the descent's evaluations and sweeps come
   from the separate kernel) are those of the caller's order, and the oracle's."""
-  n, nq, k, ef = 8000, 9000, 10, 150
+  n, nq, k = 8000, 12000, 10
   x = _data(kind, n, d, 11)
   q = _data(kind, nq, d, 12)
   ix = oracle.OracleIndex(dist).build(x, _levels(n, 0.4, 13), 8, 16, 60, 0.4)
@@ -158,18 +158,20 @@ def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, k
   ix.save(p)
   e = _engine(tmp_path, dist_type=dist, max_m=8, max_m0=16)
   e.load_index(p)
-  e.set_tunable("pair_path", 0)
-  got = {}
-  for order in (2, 0):          # 2: in order whenever the batch is more than one round of wavefronts
-    e.set_tunable("query_order", order)
-    got[order] = _device_search(e, q, k, ef)
-  for a, b in zip(got[2], got[0]):
-    assert (a == b).all()
-  o_ids, o_d, o_f, o_cnt = ix.search(q[:1500], k, ef, counters=True)
-  g_ids, g_d, g_f, stats = got[2]
-  assert (g_f[:1500] == o_f).all() and (g_ids[:1500] == o_ids).all() and (g_d[:1500] == o_d).all()
-  assert (stats[:1500, 1:] == o_cnt[:, 1:4]).all()
+  for pair, ef in ((0, 150), (2, 64)):   # one query per wavefront; two (which start level 0 at the stored entry too)
+    e.set_tunable("pair_path", pair)
+    got = {}
+    for order in (2, 0):          # 2: in order whenever the batch is more than one round of wavefronts
+      e.set_tunable("query_order", order)
+      got[order] = _device_search(e, q, k, ef)
+    for a, b in zip(got[2], got[0]):
+      assert (a == b).all()
+    o_ids, o_d, o_f, o_cnt = ix.search(q[:1500], k, ef, counters=True)
+    g_ids, g_d, g_f, stats = got[2]
+    assert (g_f[:1500] == o_f).all() and (g_ids[:1500] == o_ids).all() and (g_d[:1500] == o_d).all()
+    assert (stats[:1500, 1:] == o_cnt[:, 1:4]).all()
   e.set_tunable("query_order", 1)
+  e.set_tunable("pair_path", 1)
 
 
 def test_tight_rows_layout_and_gather_probe(oracle, tmp_path):
