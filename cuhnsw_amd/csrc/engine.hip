@@ -544,12 +544,16 @@ class Engine {
         b.live = 1;
         b.counter = d_ctl.p + 96;
         b.pool = pool;
+        // one or two of these wavefronts per CU: LDS for a candidate queue that never spills costs the first
+        // pass nothing (10 000 queries: 2.98 -> 2.87 ms; the queue of a long search outgrows 2 * ef entries)
+        if (NS > 0) b.cand_lds = std::max(a.cand_lds, 1024);
+        const LdsPlan lp_side = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, b.cand_lds, a.lcap, 0, 0, a.lean ? 0 : a.vc_bits, 0, a.lean);
         // (the first pass starts after the batch's descents when its queries are put in order: 0.1 ms per
         // 10 000 queries of the 1.18 M x 50 set; allow ten times that on top of the usual 2 ms)
         b.start_ticks += (long long)wall_clock_khz * (a.nq / 10000 + 1);
         HIP_CHECK(hipEventRecord(ev_side0, stream));
         HIP_CHECK(hipStreamWaitEvent(stream2, ev_side0, 0));
-        hipLaunchKernelGGL(kernel, dim3(side_slots), dim3(64), lp.total, stream2, ix, b);
+        hipLaunchKernelGGL(kernel, dim3(side_slots), dim3(64), lp_side.total, stream2, ix, b);
         HIP_CHECK(hipGetLastError());
         HIP_CHECK(hipEventRecord(ev_side1, stream2));
       }
