@@ -880,7 +880,15 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 // entry evicted whose key equals the bound at the group's end.  (b) An eviction finds equal largest keys: which one leaves is the heap's
 // choice, and the one that leaves stays a live candidate of hnswlib as long as that key is
 // within the bound.  The search goes on, but gives up if it comes to expand an entry with such
-// a key, or ends while such a key is still within the bound.  (c) Equal keys across
+// a key, or ends while such a key is still within the bound — except in the one case that covers most of
+// them: a single such eviction, out of exactly two equal largest keys, with fewer than the whole set asked
+// for.  Then the two twins are known (the one the set kept, the one it pushed out: the "ghost", remembered
+// with its expanded mark), hnswlib holds both in its candidate queue whichever of them its result heap kept,
+// and when their key comes up — last of all, it is the bound — it expands each of them that is not expanded
+// yet, in its heap's order.  If neither expansion has an offer accepted, the order is immaterial: nothing
+// changes but the visited marks, and the search ends there.  So the twins are expanded one after the other
+// (the ghost too, though it is not in the set), and only an accepted offer on the way gives the query up.
+// (c) Equal keys across
 // the cut at k (the result heap's choice) or among the k best (listed by label): the caller's business.
 // far: expand the farthest waiting entry instead of the closest (the reference's
 // reverse_cand); that is no hnswlib search any more, equal keys simply keep their order of
@@ -888,10 +896,13 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 template <int DT, int QR, int NS, bool BUILD>
 __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
                                                   SearchState& st, Frontier<NS>& fr, int n_seed, int lane,
-                                                  bool far = false) {
+                                                  bool far = false, bool whole_set = false) {
   const int S = row_stride(ix, level);
   int n = n_seed;
   const bool exact = !BUILD && !far;  // the outcome has to be hnswlib's
+  int ghosts = 0;                     // evictions that had equal largest keys to choose from
+  uint32_t ghost = kEmpty;            // the entry the (single) such eviction pushed out, with its expanded mark
+  bool twin_phase = false;            // the twins of that eviction are being expanded: no offer may be accepted
   bool have_tie = false;              // equal keys have met in the set
   bool in_group = false;              // the entries being expanded share one key with others still waiting
   float group_key = 0.f;
@@ -987,9 +998,20 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
         if (st.n_acc < ef || st.lower > key) {
           // an eviction out of several equal largest keys: the heap's choice decides which of
           // them stays in the result set, and the other one stays a live candidate of hnswlib
-          if (exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr)) ek_min = uni(fminf(ek_min, st.lower));
+          const bool twins = exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr);
+          const uint32_t last = twins ? (uint32_t)__builtin_amdgcn_readlane((int)fr.v[(NS > 0 ? NS : 1) - 1], 63) : kEmpty;
           const int r = frontier_insert<NS>(fr, key, id, lane);
           if (r != 2) {
+            if (twins) {
+              ek_min = uni(fminf(ek_min, st.lower));
+              ghost = last;
+              // (three or more equal largest keys, a second event, the whole set asked for: the plain rule)
+              ghosts += (frontier_max_twice<NS>(fr) || whole_set) ? 2 : 1;
+            }
+            if (exact && twin_phase) {
+              gave_up = true;  // which twin hnswlib expands first now decides whether the other one is expanded at all
+              todo = 0ull;
+            }
             have_tie = have_tie || r == 1;
             if (exact && in_group) {
               // a closer candidate turning up while a group of equal keys is being expanded would be
@@ -1013,7 +1035,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
     }
     if (gave_up) break;
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
-    const int cid = frontier_take<NS>(fr, lane, far);
+    int cid = frontier_take<NS>(fr, lane, far);
     if (exact && have_tie) {
       const float d = cid >= 0 ? frontier_key_of<NS>(fr, (uint32_t)cid) : INFINITY;
       if (in_group && d != group_key) {
@@ -1023,16 +1045,28 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
         in_group = false;
       }
       if (cid >= 0) {
-        gave_up = gave_up || d >= ek_min;
-        if (!in_group) {
+        if (d >= ek_min) {
+          // the twin the set kept: it is the set's last entry and its key is the bound
+          if (ghosts == 1 && !in_group && !frontier_open_key<NS>(fr, d)) twin_phase = true;
+          else gave_up = true;
+        }
+        if (!in_group && !twin_phase) {
           in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
           group_key = d;
           group_edge = INFINITY;
         }
-      } else {
+      } else if (!gave_up && st.n_acc >= ef && st.lower >= ek_min) {
         // an entry evicted out of equal largest keys that are still within the bound is one
         // hnswlib would go on to expand
-        gave_up = gave_up || (st.n_acc >= ef && st.lower >= ek_min);
+        if (ghosts == 1) {
+          if ((ghost & kExpanded) == 0u) {
+            cid = (int)ghost;  // the twin the set pushed out: expanded like any other, nothing of it may be accepted
+            ghost |= kExpanded;
+            twin_phase = true;
+          }
+        } else {
+          gave_up = true;
+        }
       }
     }
     if (gave_up || cid < 0) break;

@@ -316,7 +316,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     wave_sync();
     // (the flag is made wavefront-uniform explicitly and both outcomes are plain branches)
     const int how =
-        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0));
+        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0, a.k >= a.ef));
     const int T0 = st.top_size < a.k ? st.top_size : a.k;
     // Equal keys across the cut at k: which of them stays is up to the result heap, which the
     // literal search reproduces.  Equal keys among the k best: the answer lists them by label.
@@ -395,6 +395,11 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
   float lower = 0.f, maxkey = -INFINITY;
   bool have_tie = false, in_group = false, gave_up = false;
   float group_key = 0.f, group_edge = INFINITY, ek_min = INFINITY;
+  // the twins of a single eviction out of two equal largest keys (see search_level_fast)
+  int ghosts = 0;
+  uint32_t ghost = kEmpty;
+  bool twin_phase = false;
+  const bool whole_set = a.k >= ef;
   int n_dist = 0, n_hops = 0, n_dist_upper = 0, n_sweeps = 0;
   QVec<QR> qv;
 #pragma unroll
@@ -431,6 +436,7 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
           n_acc = 0; lower = 0.f; maxkey = -INFINITY;
           have_tie = false; in_group = false; gave_up = false;
           group_key = 0.f; group_edge = INFINITY; ek_min = INFINITY;
+          ghosts = 0; ghost = kEmpty; twin_phase = false;
           n_dist = 0; n_hops = 0; n_dist_upper = 0; n_sweeps = 0;
           cur = ix.enterpoint;
           phase = PP_ENTRY;
@@ -469,14 +475,26 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
         const bool open = pf_open_key<N>(fr, d, lane);
         if (on) {
           if (cid >= 0) {
-            gave_up = gave_up || d >= ek_min;
-            if (!in_group) {
+            if (d >= ek_min) {
+              // the twin the set kept: the set's last entry, its key is the bound
+              if (ghosts == 1 && !in_group && !open) twin_phase = true;
+              else gave_up = true;
+            }
+            if (!in_group && !twin_phase) {
               in_group = open;  // other waiting entries with this very key
               group_key = d;
               group_edge = INFINITY;
             }
-          } else {
-            gave_up = gave_up || (n_acc >= ef && lower >= ek_min);
+          } else if (!gave_up && n_acc >= ef && lower >= ek_min) {
+            if (ghosts == 1) {
+              if ((ghost & kExpanded) == 0u) {
+                cid = (int)ghost;  // the twin the set pushed out: expanded, nothing of it may be accepted
+                ghost |= kExpanded;
+                twin_phase = true;
+              }
+            } else {
+              gave_up = true;
+            }
           }
         }
       }
@@ -554,12 +572,26 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
         const bool acc = valid && (n_acc < ef || lower > key);
         // an eviction out of several equal largest keys: the heap's choice decides which of them stays in
         // the result set, and the other one stays a live candidate of hnswlib
+        bool twins = false;
+        uint32_t last = kEmpty;
         if (wave_any(acc && have_tie && n_acc >= ef)) {
-          const bool twice = pf_max_twice<N>(fr, lane);
-          if (acc && have_tie && n_acc >= ef && twice) ek_min = fminf(ek_min, lower);
+          twins = acc && have_tie && n_acc >= ef && pf_max_twice<N>(fr, lane);
+          last = (uint32_t)__builtin_bit_cast(int, half_last(__builtin_bit_cast(float, (int)fr.v[N - 1]), lane));
         }
         const int r = pf_insert<N>(fr, key, id, acc, lane);
         const bool ins = acc && r != 2;
+        if (wave_any(ins && twins)) {
+          const bool still = pf_max_twice<N>(fr, lane);
+          if (ins && twins) {
+            ek_min = fminf(ek_min, lower);
+            ghost = last;
+            ghosts += (still || whole_set) ? 2 : 1;  // three equal largest keys, a second event, the whole set asked for
+          }
+        }
+        if (ins && twin_phase) {
+          gave_up = true;  // which twin hnswlib expands first now decides whether the other one is expanded at all
+          todo = 0u;
+        }
         have_tie = have_tie || (ins && r == 1);
         if (ins && in_group) {
           // a closer candidate turning up while a group of equal keys is being expanded would be expanded
