@@ -166,6 +166,11 @@ def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, k
       got[order] = _device_search(e, q, k, ef)
     for a, b in zip(got[2], got[0]):
       assert (a == b).all()
+    e.set_tunable("concurrent_literal", 0)   # the literal pass after the first one instead of beside it
+    e.set_tunable("query_order", 2)
+    for a, b in zip(_device_search(e, q, k, ef), got[0]):
+      assert (a == b).all()
+    e.set_tunable("concurrent_literal", 1)
     o_ids, o_d, o_f, o_cnt = ix.search(q[:1500], k, ef, counters=True)
     g_ids, g_d, g_f, stats = got[2]
     assert (g_f[:1500] == o_f).all() and (g_ids[:1500] == o_ids).all() and (g_d[:1500] == o_d).all()
