@@ -875,9 +875,13 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 // none exists under any order, the whole group is expanded back to back and the set afterwards
 // is the ef smallest of old set and offers either way — up to entries whose key equals the
 // bound the set ends up with: whether such an offer is accepted or turned away, and which of
-// several such entries is evicted, does depend on the order.  So a key below d during the
-// group gives the query up, and so does a group during which an offer was turned away or an
-// entry evicted whose key equals the bound at the group's end.  (b) An eviction finds equal largest keys: which one leaves is the heap's
+// several such entries is evicted, does depend on the order.  So a group during which an offer was turned
+// away or an entry evicted whose key equals the bound at the group's end gives the query up.  A key below d
+// turning up during the group does not by itself: such a candidate (and whatever closer ones it leads to) is
+// expanded before the rest of the group under any order, and by the same argument the set after the last
+// member is the same — provided every member does get expanded under any order, i.e. the bound is still at
+// or above d when the group is through and no member was pushed out of the set before its turn; a second group
+// of equal keys among those closer candidates is not followed (given up).  (b) An eviction finds equal largest keys: which one leaves is the heap's
 // choice, and the one that leaves stays a live candidate of hnswlib as long as that key is
 // within the bound.  The search goes on, but gives up if it comes to expand an entry with such
 // a key, or ends while such a key is still within the bound — except in the one case that covers most of
@@ -999,12 +1003,15 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
           // an eviction out of several equal largest keys: the heap's choice decides which of
           // them stays in the result set, and the other one stays a live candidate of hnswlib
           const bool twins = exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr);
-          const uint32_t last = twins ? (uint32_t)__builtin_amdgcn_readlane((int)fr.v[(NS > 0 ? NS : 1) - 1], 63) : kEmpty;
+          // the entry a full set is about to push out, where somebody will ask for it
+          const uint32_t evicted = (twins || (exact && in_group && st.n_acc >= ef && st.lower == group_key))
+                                       ? (uint32_t)__builtin_amdgcn_readlane((int)fr.v[(NS > 0 ? NS : 1) - 1], 63)
+                                       : kEmpty;
           const int r = frontier_insert<NS>(fr, key, id, lane);
           if (r != 2) {
             if (twins) {
               ek_min = uni(fminf(ek_min, st.lower));
-              ghost = last;
+              ghost = evicted;
               // (three or more equal largest keys, a second event, the whole set asked for: the plain rule)
               ghosts += (frontier_max_twice<NS>(fr) || whole_set) ? 2 : 1;
             }
@@ -1013,14 +1020,12 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
               todo = 0ull;
             }
             have_tie = have_tie || r == 1;
-            if (exact && in_group) {
-              // a closer candidate turning up while a group of equal keys is being expanded would be
-              // expanded before or after the rest of the group depending on the heap's order
-              if (key < group_key) {
+            if (exact && in_group && st.n_acc >= ef) {
+              group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
+              // a member of the group pushed out before its turn: with another order it would have been expanded
+              if (st.lower == group_key && (evicted & kExpanded) == 0u) {
                 gave_up = true;
                 todo = 0ull;
-              } else if (st.n_acc >= ef) {
-                group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
               }
             }
             st.n_acc = uni(st.n_acc + 1);
@@ -1038,10 +1043,15 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
     int cid = frontier_take<NS>(fr, lane, far);
     if (exact && have_tie) {
       const float d = cid >= 0 ? frontier_key_of<NS>(fr, (uint32_t)cid) : INFINITY;
-      if (in_group && d != group_key) {
+      if (in_group && cid >= 0 && d < group_key) {
+        // a closer candidate turned up inside the group: it is expanded before the rest of the group under any
+        // order.  A group within the group is not followed.
+        gave_up = frontier_open_key<NS>(fr, d);
+      } else if (in_group && d != group_key) {
         // the group is through.  With another order of its members an offer or an entry whose
-        // key equals the bound reached now could have ended up on the other side of it.
-        gave_up = st.n_acc >= ef && group_edge == st.lower;
+        // key equals the bound reached now could have ended up on the other side of it; and with the bound
+        // below the group's key a member popped late would not have been expanded at all.
+        gave_up = st.n_acc >= ef && (group_edge == st.lower || st.lower < group_key);
         in_group = false;
       }
       if (cid >= 0) {

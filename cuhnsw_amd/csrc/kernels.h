@@ -466,13 +466,18 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
       if (wave_any(phase == PP_SEARCH && have_tie)) {
         const bool on = phase == PP_SEARCH && have_tie;
         const float d = cid >= 0 ? pf_key_of<N>(fr, (uint32_t)(cid >= 0 ? cid : 0), lane) : INFINITY;
-        if (on && in_group && d != group_key) {
+        const bool open = pf_open_key<N>(fr, d, lane);
+        if (on && in_group && cid >= 0 && d < group_key) {
+          // a closer candidate inside the group: expanded before the rest of it under any order; a group
+          // within the group is not followed
+          gave_up = open;
+        } else if (on && in_group && d != group_key) {
           // the group is through: with another order of its members an offer or an entry whose key equals
-          // the bound reached now could have ended up on the other side of it
-          gave_up = n_acc >= ef && group_edge == lower;
+          // the bound reached now could have ended up on the other side of it, and with the bound below the
+          // group's key a member popped late would not have been expanded at all
+          gave_up = n_acc >= ef && (group_edge == lower || lower < group_key);
           in_group = false;
         }
-        const bool open = pf_open_key<N>(fr, d, lane);
         if (on) {
           if (cid >= 0) {
             if (d >= ek_min) {
@@ -573,7 +578,7 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
         // an eviction out of several equal largest keys: the heap's choice decides which of them stays in
         // the result set, and the other one stays a live candidate of hnswlib
         bool twins = false;
-        uint32_t last = kEmpty;
+        uint32_t last = kEmpty;  // the entry a full set is about to push out
         if (wave_any(acc && have_tie && n_acc >= ef)) {
           twins = acc && have_tie && n_acc >= ef && pf_max_twice<N>(fr, lane);
           last = (uint32_t)__builtin_bit_cast(int, half_last(__builtin_bit_cast(float, (int)fr.v[N - 1]), lane));
@@ -593,14 +598,12 @@ __global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevInde
           todo = 0u;
         }
         have_tie = have_tie || (ins && r == 1);
-        if (ins && in_group) {
-          // a closer candidate turning up while a group of equal keys is being expanded would be expanded
-          // before or after the rest of the group depending on the heap's order
-          if (key < group_key) {
+        if (ins && in_group && n_acc >= ef) {
+          group_edge = fminf(group_edge, lower);  // the entry this insert evicted
+          // a member of the group pushed out before its turn: with another order it would have been expanded
+          if (lower == group_key && (last & kExpanded) == 0u) {
             gave_up = true;
             todo = 0u;
-          } else if (n_acc >= ef) {
-            group_edge = fminf(group_edge, lower);  // the entry this insert evicted
           }
         }
         if (valid && !acc && in_group) group_edge = fminf(group_edge, key);

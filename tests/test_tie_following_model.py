@@ -36,8 +36,6 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
       last = list(S[-1])
       if any(e[0] == key for e in S):
         have_tie = True
-      if in_group and key < group_key:
-        return None                           # a closer candidate inside a group of equal keys
       pos = len(S)
       while pos > 0 and S[pos - 1][0] > key:
         pos -= 1
@@ -45,6 +43,8 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
       if len(S) > ef:
         if in_group:
           group_edge = min(group_edge, S[-1][0])
+          if S[-1][0] == group_key and not S[-1][2]:
+            return None                       # a member of the group pushed out before its turn
         S.pop()
       if twins:
         ek_min = min(ek_min, last[0])
@@ -55,10 +55,16 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
         return None                           # which twin goes first now decides whether the other is expanded at all
     pick = next((i for i, e in enumerate(S) if not e[2]), -1)
     d = S[pick][0] if pick >= 0 else INF
-    if in_group and d != group_key:
+    if in_group and pick >= 0 and d < group_key:
+      # a closer candidate turned up inside the group: it is expanded before the rest of the group under
+      # any order; a group within the group is not followed
+      if any((not e[2]) and e[0] == d for i, e in enumerate(S) if i != pick):
+        return None
+    elif in_group and d != group_key:
       # the group is through: with another order of its members an offer or an entry whose key
-      # equals the bound reached now could have ended up on the other side of it
-      if len(S) >= ef and group_edge == S[-1][0]:
+      # equals the bound reached now could have ended up on the other side of it, and with the bound
+      # below the group's key a member popped late would not have been expanded at all
+      if len(S) >= ef and (group_edge == S[-1][0] or S[-1][0] < group_key):
         return None
       in_group = False
     if pick < 0:
