@@ -124,6 +124,7 @@ class Engine {
   int hnswlib_dist = 0;
   int spin_limit_override = -1;  // polls a waiting literal wavefront may spend (-1 = automatic)
   int side_per_cu = 0;         // its wavefronts per CU (0 = from the share of queries the last search gave up)
+  bool share_known = false;               // last_repeat_share comes from a search of this index
   double last_repeat_share = 0.0;         // its wavefronts per CU
   int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
@@ -516,8 +517,11 @@ class Engine {
       const int per_cu = side_per_cu > 0 ? side_per_cu : (last_repeat_share < 0.02 ? 1 : 2);
       if (side) {
         side_slots = std::min(num_cus * per_cu, a.nq);
+        // an index that hands over next to nothing (the last search: under one query in a thousand) gets one
+        // literal wavefront per four CUs, and the first pass the room of the others
+        if (side_per_cu <= 0 && share_known && last_repeat_share < 0.001) side_slots = std::min(std::max(num_cus / 4, 1), a.nq);
         ensure_pool(std::max(side_slots, 1), glob_cap, 2 * glob_cap);
-        slots = std::max(num_cus, slots - num_cus * per_cu);  // leave the literal wavefronts their room
+        slots = std::max(num_cus, slots - std::min(side_slots, num_cus * per_cu));  // leave the literal wavefronts their room
       }
       if (max_slots_override > 0) slots = max_slots_override;
       if (first_pass_waves > 0) slots = std::min(slots, first_pass_waves * num_cus);
@@ -587,6 +591,7 @@ class Engine {
       HIP_CHECK(hipStreamSynchronize(stream));
       n_literal = last_repeats = ctl[32];
       last_repeat_share = (double)n_literal / a.nq;
+      share_known = true;
       // an index whose distances tie all the time (integer-valued data) sends most queries
       // through both passes: stop trying the sorted set on it
       if (a.nq >= 256 && (long long)n_literal * 3 > a.nq) fast_suspended = true;
@@ -973,6 +978,7 @@ class Engine {
     last_build_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     have_graph = true;
     fast_suspended = false;
+    share_known = false;
     host_links_stale = true;
   }
 
@@ -1017,6 +1023,7 @@ class Engine {
     host = std::move(fresh);
     have_data = have_levels = have_graph = true;
     fast_suspended = false;
+    share_known = false;
     host_links_stale = false;
     if (has_device) {
       upload_vectors();
