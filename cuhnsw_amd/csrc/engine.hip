@@ -473,8 +473,14 @@ class Engine {
     int n_literal = a.nq;
     bool answered = false;
     // A batch that fits the machine in one round of literal wavefronts is latency-bound: two
-    // passes would only add the second pass's latency to the first's.
-    if (NS > 0 && a.fast_path && a.fc_bits > 0 && (a.fast_path > 1 || a.nq > lit_slots)) {  // (reverse_cand: fast_path is 2)
+    // passes would only add the second pass's latency to the first's — where the literal search has its exact
+    // bitmaps (100 000 points, 1 000 queries: 1.06 ms literal only; 0.75 ms through the first pass, but 1.76 when
+    // one query is handed over at its end).  Where the bitmaps do not fit the L2 and the literal search runs on the
+    // sorted set with the LDS filter, the first pass is the same search without the literal candidate queue, and
+    // the faster one even with a hand-over (1.18 M points, 2 000 queries: 1.73 against 2.36 ms; 1 M x 960, 1 000
+    // queries: 5.33 against 5.95 ms).
+    if (NS > 0 && a.fast_path && a.fc_bits > 0 &&
+        (a.fast_path > 1 || a.nq > lit_slots || (a.lean && a.nq > 1))) {  // (reverse_cand: fast_path is 2)
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
       auto fast_kernel = search_fast_kernel<DT, QR, NS>;
