@@ -130,7 +130,7 @@ class Engine {
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   int first_pass_waves = 0;  // wavefronts per CU of the first pass (0 = as many as fit)
   int pair_path = 1;       // first pass with two queries per wavefront where the shapes allow it (0: one per wavefront)
-  int query_order = 1;     // first pass of two or more rounds of wavefronts: longest queries first (0: caller's order)
+  int query_order = 1;     // first pass of 1.5 to 32 rounds of wavefronts: longest queries first (0: caller's order)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
   bool storage_half = false;  // vectors live in HBM as fp16 (set before set_data / load_index)
@@ -536,14 +536,15 @@ class Engine {
       HIP_CHECK(hipMemsetAsync(d_redo.p, 0xFF, (size_t)a.nq * sizeof(int), stream));
       // (every allocation before the literal pass is launched: growing a buffer frees the old one, and
       // hipFree waits for the device, on which that pass would be waiting for the first pass to start)
-      // (from two rounds of wavefronts on — 1.18 M x 50, 40 000 queries: 8.25 -> 7.41 ms; at 1.45 rounds, 10 000
-      // queries, the first pass alone gains, 2.46-2.76 -> 2.14 ms, but its heavy queries then hand over late and the
-      // batch ends no earlier, 3.2 against 3.0-3.1 ms; query_order = 2 puts any batch of more than one round in order)
+      // (from one and a half rounds of wavefronts on — 1.18 M x 50, 40 000 queries: 8.25 -> 7.41 ms; eight draws of
+      // 12 000 queries, 1.7 rounds: 3.10 -> 2.85 ms on average; of 10 000, 1.4 rounds: 2.92 and 2.96 — the first
+      // pass alone gains, 2.8 -> 2.2 ms, but the one query in ten thousand that is handed over then tends to be
+      // one that ends last; query_order = 2 puts any batch of more than one round in order)
       const long long resident = pair ? 2LL * slots : slots;  // queries at work at a time
       // (and up to 32 rounds: what the order saves is part of one round, what the separate descents cost grows
       // with the batch — 1 000 000 queries, 145 rounds: 211.7 against 201.9 ms in the caller's order)
       const bool in_order = query_order && (query_order > 1 ? a.nq > resident
-                                                             : a.nq >= 2 * resident && a.nq <= 32 * resident);
+                                                             : 2 * a.nq >= 3 * resident && a.nq <= 32 * resident);
       if (in_order) {
         d_entry.reserve((size_t)a.nq);
         d_order.reserve((size_t)a.nq);

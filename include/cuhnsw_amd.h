@@ -161,7 +161,7 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   batch exceeds one round of resident wavefronts, literal queues for the queries
  *                   that met equal distances (default); 2 = first pass whatever the batch size
  *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
- *   "query_order"   1 (default) = a search batch of two or more rounds of wavefronts does its upper-level descents
+ *   "query_order"   1 (default) = a search batch of 1.5 to 32 rounds of wavefronts does its upper-level descents
  *                   first and takes its queries by descending distance of their level-0 entry point (the longest
  *                   searches first: a launch ends when its last query does); 2 = from more than one round on;
  *                   0 = in the caller's order.  Same answers and counters either way.
