@@ -576,14 +576,21 @@ class Engine {
         a.order = d_order.p;
         a.order_hist = d_order_hist.p;
         HIP_CHECK(hipMemsetAsync(d_order_hist.p, 0, (size_t)kOrderBuckets * sizeof(int), stream));
-        auto k_entry = entry_kernel<DT, QR>;
-        const size_t entry_lds = plan_fast_lds(QR, ix.Dp, a.lcap, 0).total;
-        const int entry_grid = std::max(1, std::min(a.nq, resident_slots(k_entry, entry_lds)));
-        hipLaunchKernelGGL(k_entry, dim3(entry_grid), dim3(64), entry_lds, stream, ix, a);
+        if constexpr (QR == 1 || QR == 2) {
+          // four queries per wavefront, one per group of 16 lanes (40 000 queries: 0.28 -> 0.16 ms)
+          auto k_entry = entry4_kernel<DT, QR>;
+          const int entry_grid = std::max(1, std::min((a.nq + 3) / 4, resident_slots(k_entry, 0)));
+          hipLaunchKernelGGL(k_entry, dim3(entry_grid), dim3(64), 0, stream, ix, a);
+        } else {
+          auto k_entry = entry_kernel<DT, QR>;
+          const size_t entry_lds = plan_fast_lds(QR, ix.Dp, a.lcap, 0).total;
+          const int entry_grid = std::max(1, std::min(a.nq, resident_slots(k_entry, entry_lds)));
+          hipLaunchKernelGGL(k_entry, dim3(entry_grid), dim3(64), entry_lds, stream, ix, a);
+        }
         HIP_CHECK(hipGetLastError());
         hipLaunchKernelGGL(order_prefix_kernel, dim3(1), dim3(1024), 0, stream, d_order_hist.p);
         HIP_CHECK(hipGetLastError());
-        hipLaunchKernelGGL(order_scatter_kernel, dim3((unsigned)((a.nq + 255) / 256)), dim3(256), 0, stream, d_entry.p,
+        hipLaunchKernelGGL(order_scatter_kernel, dim3((unsigned)((a.nq + 1023) / 1024)), dim3(1024), 0, stream, d_entry.p,
                            a.nq, d_order_hist.p, d_order.p);
         HIP_CHECK(hipGetLastError());
       }

@@ -230,6 +230,96 @@ __global__ void __launch_bounds__(64) entry_kernel(DevIndex ix, SearchArgs a) {
     wave_sync();
   }
 }
+// The same descents, FOUR queries per wavefront, one per group of 16 lanes (rows of up to 128 elements: the
+// query in one or two float4 registers per lane).  A descent is a chain of dependent fetches with a dozen
+// evaluations each; on its own in a kernel it is bound by their latency, and a group of 16 lanes is what one
+// evaluation occupies anyway: the four groups walk their own queries' levels side by side, each evaluating
+// the ids of its current link row one after the other (eight or sixteen rows in flight per lane), with the same
+// arithmetic, the same strict first minimum and the same counters as `descend`.
+template <int DT, int QR, bool HALF>
+__device__ __forceinline__ float entry4_key(const void* rows, uint32_t rowlen, uint32_t used, const QVec<QR>& qv,
+                                            uint32_t id, int sub) {
+  constexpr int R = QR > 0 ? QR : 1;
+  const uint64_t first = (uint64_t)id * rowlen;
+  float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
+#pragma unroll
+  for (int k = 0; k < R; ++k) {
+    const uint32_t c = sub + 16 * k;
+    const uint64_t at = first + (c < used ? c : 0);  // (as in dist_pass: one unconditional load, padding replaced)
+    const float4 t = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
+    const float4 v = (DT == DIST_DOT || k < R / 2 || c < used) ? t : qv.q[k];
+    acc4<DT>(qv.q[k], v, ax, ay, az, aw);
+  }
+  return finish16<DT, false>(ax, ay, az, aw);
+}
+template <int DT, int QR, bool HALF>
+__device__ __forceinline__ void entry4_body(const DevIndex& ix, const SearchArgs& a) {
+  const int lane = threadIdx.x, g = lane >> 4, sub = lane & 15;
+  const uint32_t rowlen = (uint32_t)ix.Dp >> 2, used = (uint32_t)(ix.D + 3) >> 2;
+  const void* rows = ix.vectors;
+  for (int q0 = blockIdx.x * 4; q0 < a.nq; q0 += gridDim.x * 4) {
+    const int qi = q0 + g;
+    const bool have = qi < a.nq;
+    QVec<QR> qv;
+    load_query<QR>(qv, nullptr, a.q + (size_t)(have ? qi : 0) * ix.D, ix.D, ix.Dp, lane);
+    uint32_t cur = ix.enterpoint;
+    float dcur = entry4_key<DT, QR, HALF>(rows, rowlen, used, qv, cur, sub);
+    int level = ix.maxlevel;
+    bool active = have && level > 0;
+    int sweeps = 0, evals = 0;
+    while (__ballot(active) != 0ull) {
+      const uint32_t* row = ix.linksU + (size_t)(ix.upper_off[active ? cur : ix.enterpoint] + (active ? level : 1) - 1) * ix.SU;
+      float best = INFINITY;
+      uint32_t best_id = cur;
+      int n = 0;
+      for (int base = 0; base < ix.SU; base += 16) {
+        const uint32_t got = row[base + sub < ix.SU ? base + sub : 0];
+        const uint32_t id = (active && base + sub < ix.SU) ? got : kEmpty;
+        const unsigned long long valid = __ballot(id != kEmpty);
+        n += __popc((uint32_t)(valid >> (16 * g)) & 0xFFFFu);
+        constexpr int B = QR == 1 ? 16 : 8;  // rows in flight per lane: 16 float4 registers' worth
+#pragma unroll
+        for (int p0 = 0; p0 < 16; p0 += B) {
+          if (((valid >> p0) & (0x0001000100010001ull * ((1u << B) - 1u))) == 0ull) continue;  // no id in these slots
+          uint32_t ids[B];
+          float keys[B];
+#pragma unroll
+          for (int j = 0; j < B; ++j) ids[j] = (uint32_t)__shfl((int)id, 16 * g + p0 + j, 64);
+#pragma unroll
+          for (int j = 0; j < B; ++j)
+            keys[j] = entry4_key<DT, QR, HALF>(rows, rowlen, used, qv, ids[j] != kEmpty ? ids[j] : cur, sub);
+#pragma unroll
+          for (int j = 0; j < B; ++j)
+            if (ids[j] != kEmpty && keys[j] < best) {  // strictly closer: the first occurrence of the minimum wins
+              best = keys[j];
+              best_id = ids[j];
+            }
+        }
+      }
+      if (active) {
+        sweeps += 1;
+        evals += n;
+        if (n > 0 && best < dcur) {
+          dcur = best;
+          cur = best_id;  // and sweep again on this level
+        } else {
+          level -= 1;
+          active = level > 0;
+        }
+      }
+    }
+    if (have && sub == 0) {
+      const uint32_t bits = __float_as_uint(dcur);
+      a.entry[qi] = make_uint4(cur, bits, (uint32_t)evals, (uint32_t)sweeps);
+      atomicAdd(a.order_hist + order_bucket(bits), 1);
+    }
+  }
+}
+template <int DT, int QR>
+__global__ void __launch_bounds__(64) entry4_kernel(DevIndex ix, SearchArgs a) {
+  if (uni(ix.half) != 0) entry4_body<DT, QR, true>(ix, a);
+  else entry4_body<DT, QR, false>(ix, a);
+}
 // counters -> first position of every bucket (exclusive prefix sum; one workgroup of 1024)
 __global__ void __launch_bounds__(1024) order_prefix_kernel(int* hist) {
   __shared__ int part[1024];
@@ -257,9 +347,26 @@ __global__ void __launch_bounds__(1024) order_prefix_kernel(int* hist) {
     run += local[i];
   }
 }
-__global__ void __launch_bounds__(256) order_scatter_kernel(const uint4* entry, int nq, int* cursor, int* order) {
-  const int qi = blockIdx.x * 256 + threadIdx.x;
-  if (qi < nq) order[atomicAdd(cursor + order_bucket(entry[qi].y), 1)] = qi;
+__global__ void __launch_bounds__(1024) order_scatter_kernel(const uint4* entry, int nq, int* cursor, int* order) {
+  // The keys of a batch fall into a few dozen buckets: a workgroup ranks its 1024 queries in LDS and takes one
+  // range per bucket it met from the global cursors (the order inside a bucket is free).
+  __shared__ int cnt[kOrderBuckets];
+  const int t = threadIdx.x;
+  for (int i = t; i < kOrderBuckets; i += 1024) cnt[i] = 0;
+  __syncthreads();
+  const int qi = blockIdx.x * 1024 + t;
+  int bucket = 0, rank = 0;
+  if (qi < nq) {
+    bucket = order_bucket(entry[qi].y);
+    rank = atomicAdd(&cnt[bucket], 1);
+  }
+  __syncthreads();
+  for (int i = t; i < kOrderBuckets; i += 1024) {
+    const int c = cnt[i];
+    if (c > 0) cnt[i] = atomicAdd(cursor + i, c);
+  }
+  __syncthreads();
+  if (qi < nq) order[cnt[bucket] + rank] = qi;
 }
 
 // First pass of a search batch: every query on the sorted set in registers (ef < 64*NS).
