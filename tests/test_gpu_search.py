@@ -145,18 +145,26 @@ def test_two_queries_per_wavefront_equal_one_per_wavefront(oracle, tmp_path, nam
   e.set_tunable("pair_path", 1)
 
 
-@pytest.mark.parametrize("kind,d,dist", [("gauss", 50, "dot"), ("int", 24, "l2")], ids=["dot50", "l2_int_ties"])
-def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, kind, d, dist):
-  """A batch of several rounds of wavefronts does its upper-level descents first and takes its queries by
-  descending entry distance.  Answers, found counts and every counter (the descent's evaluations and sweeps come
-  from the separate kernel) are those of the caller's order, and the oracle's."""
+@pytest.mark.parametrize("kind,d,dist,max_m,half", [
+    ("gauss", 50, "dot", 8, False), ("int", 24, "l2", 8, False),
+    ("gauss_raw", 100, "l2", 20, False),   # two register chunks per lane; upper-level rows longer than 16 ids
+    ("int", 128, "l2", 16, True),          # fp16 rows (integers below 2048 are exact in fp16), full upper-level rows
+    ("gauss", 160, "dot", 8, False),       # rows too long for registers: the descents one query per wavefront
+], ids=["dot50", "l2_int_ties", "l2_100_m20", "l2_128_fp16", "dot160"])
+def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, kind, d, dist, max_m, half):
+  """A batch of several rounds of wavefronts does its upper-level descents first (four queries per wavefront
+  where the rows fit registers) and takes its queries by descending entry distance.  Answers, found counts and
+  every counter (the descent's evaluations and sweeps come from the separate kernel) are those of the caller's
+  order, and the oracle's."""
   n, nq, k = 8000, 12000, 10
   x = _data(kind, n, d, 11)
   q = _data(kind, nq, d, 12)
-  ix = oracle.OracleIndex(dist).build(x, _levels(n, 0.4, 13), 8, 16, 60, 0.4)
+  ix = oracle.OracleIndex(dist).build(x, _levels(n, 0.4, 13), max_m, 2 * max_m, 60, 0.4)
   p = str(tmp_path / "i.idx")
   ix.save(p)
-  e = _engine(tmp_path, dist_type=dist, max_m=8, max_m0=16)
+  e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=2 * max_m)
+  if half:
+    e.set_tunable("fp16_storage", 1)
   e.load_index(p)
   for pair, ef in ((0, 150), (2, 64)):   # one query per wavefront; two (which start level 0 at the stored entry too)
     e.set_tunable("pair_path", pair)
