@@ -127,7 +127,10 @@ def main():
   ap.add_argument("--pair-path", type=int, default=1, choices=[0, 1, 2],
                   help="0 = never two queries per wavefront in the first pass, 2 = wherever the shapes allow it")
   ap.add_argument("--query-order", type=int, default=1, choices=[0, 1, 2],
-                  help="0 = queries in the caller's order, 1 = longest first from two rounds of wavefronts on, 2 = from one")
+                  help="0 = queries in the caller's order, 1 = longest first from one to one and a half rounds of wavefronts on, 2 = from one")
+  ap.add_argument("--trails", type=int, default=1, choices=[0, 1, 2],
+                  help="0 = the literal pass searches handed-over queries from the entry point, 1 = from the first pass's "
+                       "trail in batches of up to two rounds of wavefronts (default), 2 = in every batch")
   ap.add_argument("--no-large", action="store_true", help="skip the extra 4x batch (profiling runs)")
   ap.add_argument("--profile", action="store_true",
                   help="profiling run: only searches of the default path are launched (no literal-only counting pass, "
@@ -197,6 +200,7 @@ def main():
   build_s = eng.last_build_seconds
   eng.set_tunable("pair_path", args.pair_path)
   eng.set_tunable("query_order", args.query_order)
+  eng.set_tunable("trails", args.trails)
 
   # exact top-k on the GPU (harness only) for recall.  Scores are produced in blocks of at most
   # 2^28 elements (1 GiB): larger matmul outputs came back with wrong entries on this stack.

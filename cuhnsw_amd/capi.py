@@ -17,7 +17,7 @@ SYMBOLS = [
     "cuhnsw_max_level", "cuhnsw_enter_point", "cuhnsw_has_device",
     "cuhnsw_last_build_seconds", "cuhnsw_last_search_repeats", "cuhnsw_set_tunable",
     "cuhnsw_search_knn_device_noalloc", "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
-    "cuhnsw_last_build_counters", "cuhnsw_debug_gather_probe",
+    "cuhnsw_last_build_counters", "cuhnsw_debug_gather_probe", "cuhnsw_last_search_trails",
 ]
 
 _lib = None
@@ -56,6 +56,7 @@ def load():
   l.cuhnsw_last_build_seconds.argtypes = [vp]
   l.cuhnsw_last_build_seconds.restype = cd
   l.cuhnsw_last_search_repeats.argtypes = [vp]
+  l.cuhnsw_last_search_trails.argtypes = [vp]
   l.cuhnsw_set_tunable.argtypes = [vp, ctypes.c_char_p, cd]
   _lib = l
   return l
@@ -175,4 +176,5 @@ class Engine:
   enter_point = property(lambda s: s._l.cuhnsw_enter_point(s._h))
   last_build_seconds = property(lambda s: s._l.cuhnsw_last_build_seconds(s._h))
   last_search_repeats = property(lambda s: s._l.cuhnsw_last_search_repeats(s._h))
+  last_search_trails = property(lambda s: s._l.cuhnsw_last_search_trails(s._h))
   last_build_dropped_links = property(lambda s: s._l.cuhnsw_last_build_dropped_links(s._h))

@@ -861,6 +861,65 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
   }
 }
 
+// The trail of a sorted-set search: the entries it accepted, hop by hop, wherever its course is certainly
+// hnswlib's own.  A query that is given up afterwards is not searched again from its entry point: the
+// literal pass takes the accepted entries of those hops from the trail — no link rows, no vectors, no
+// arithmetic, only its queue and set operations in hnswlib's order — and searches on from where the trail
+// ends.  One 16-byte record per accepted entry: (expanded node, accepted node, key bits, number of the hop);
+// hops without an accepted entry leave none.  While equal keys wait side by side (a group that is followed
+// through) the order of expansion may differ from hnswlib's and with it what each hop accepts: those hops are
+// not recorded, two markers (kTrailOwn from hop h on, kTrailBack from hop h on) tell the literal pass to make
+// them itself, in its own order; after such a group the set, the bound and the nodes met are the same again
+// under either order, and so is what every later hop accepts.  The trail ends for good when the twins of an
+// eviction come up (a node outside the set is expanded there).
+constexpr uint32_t kTrailOwn = 0xFFFFFFFFu;
+constexpr uint32_t kTrailBack = 0xFFFFFFFEu;
+struct Trail {
+  uint4* rec = nullptr;  // this search's records, or null: no trail is kept
+  int cap = 0;
+  int n = 0;         // records written; -1: the trail outgrew its buffer and is void
+  int hops = 0;      // expansions the trail covers (all of them completed)
+  int n_dist = 0;    // evaluations up to there
+  bool on = false;   // still recording
+  bool own = false;  // inside a stretch the literal pass makes itself
+};
+__device__ __forceinline__ void trail_mark(Trail& tr, uint32_t kind, int hop, int lane) {
+  if (tr.on) {
+    if (tr.n + 1 > tr.cap) {
+      tr.on = false;
+      tr.n = -1;
+    } else {
+      if (lane == 0) tr.rec[tr.n] = make_uint4(kind, 0u, 0u, (uint32_t)hop);
+      tr.n += 1;
+      tr.own = kind == kTrailOwn;
+    }
+  }
+}
+__device__ __forceinline__ void trail_hop(Trail& tr, unsigned long long accepted, int cid, int hop, uint32_t my_id,
+                                          float my_key, int lane) {
+  if (tr.on && !tr.own && accepted != 0ull && cid >= 0) {
+    const int cnt = __popcll(accepted);
+    if (tr.n + cnt > tr.cap) {
+      tr.on = false;
+      tr.n = -1;
+    } else {
+      if ((accepted >> lane) & 1ull) {
+        const int at = tr.n + __popcll(accepted & ((1ull << lane) - 1ull));
+        tr.rec[at] = make_uint4((uint32_t)cid, my_id, __float_as_uint(my_key), (uint32_t)hop);
+      }
+      tr.n += cnt;
+    }
+  }
+}
+// the trail ends here: `hops` expansions are complete
+__device__ __forceinline__ void trail_stop(Trail& tr, int hops, int n_dist) {
+  if (tr.on) {
+    tr.on = false;
+    tr.hops = hops;
+    tr.n_dist = n_dist;
+  }
+}
+
 // Best-first search of one level on the sorted set (needs the LDS tag filter).  On entry
 // s.nbuf[0..n_seed) holds the seeds, already entered into the filter.  Returns 0: fr holds the
 // result (st.top_size entries, ascending), all keys were distinct; 2: the same, but equal keys
@@ -900,10 +959,14 @@ __device__ __forceinline__ void visit_lossy_single(Scratch& s, uint32_t id, int 
 template <int DT, int QR, int NS, bool BUILD>
 __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
                                                   SearchState& st, Frontier<NS>& fr, int n_seed, int lane,
-                                                  bool far = false, bool whole_set = false) {
+                                                  bool far = false, bool whole_set = false, Trail* trail = nullptr) {
   const int S = row_stride(ix, level);
   int n = n_seed;
   const bool exact = !BUILD && !far;  // the outcome has to be hnswlib's
+  Trail no_trail;
+  Trail& tr = trail ? *trail : no_trail;
+  unsigned long long accepted = 0ull;  // offers of the current hop that entered the set
+  int hop_cid = -1;                    // the node the current hop expanded (-1: the seeds)
   int ghosts = 0;                     // evictions that had equal largest keys to choose from
   uint32_t ghost = kEmpty;            // the entry the (single) such eviction pushed out, with its expanded mark
   bool twin_phase = false;            // the twins of that eviction are being expanded: no offer may be accepted
@@ -939,6 +1002,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
           for (int t = 0; t < (NS > 0 ? NS : 1); ++t) eq = eq || fr.k[t] == key;
           if (__ballot(eq) == 0ull) {
             frontier_insert_distinct<NS>(fr, key, id);
+            accepted |= 1ull << j;
             st.n_acc = st.n_acc + 1;
             if (st.n_acc < ef) {
               st.maxkey = uni(fmaxf(st.maxkey, key));
@@ -959,18 +1023,24 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
         }
       }
       if (resume_at >= 0) break;
+      trail_hop(tr, accepted, hop_cid, st.n_hops, my_id, my_key, lane);
+      accepted = 0ull;
       st.top_size = st.n_acc < ef ? st.n_acc : ef;
       const int cid = frontier_take<NS>(fr, lane, false);
       if (cid < 0) {
         finished = true;
         break;
       }
+      hop_cid = cid;
       st.n_hops += 1;
       wave_sync();
       n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
       wave_sync();
     }
-    if (finished) return 0;
+    if (finished) {
+      trail_stop(tr, st.n_hops, st.n_dist);
+      return 0;
+    }
   }
   while (true) {
     if (resume_at < 0) {
@@ -1009,6 +1079,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
                                        : kEmpty;
           const int r = frontier_insert<NS>(fr, key, id, lane);
           if (r != 2) {
+            accepted |= 1ull << j;
             if (twins) {
               ek_min = uni(fminf(ek_min, st.lower));
               ghost = evicted;
@@ -1037,10 +1108,16 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
         }
       }
       if (gave_up) base = n;  // leave the outer loop as well
+      else trail_hop(tr, accepted, hop_cid, st.n_hops, my_id, my_key, lane);  // (a trail is kept for rows of one pass only)
+      accepted = 0ull;
     }
-    if (gave_up) break;
+    if (gave_up) {
+      trail_stop(tr, st.n_hops - 1, st.n_dist);  // (a trail still recording here: the hop under way is not on it)
+      break;
+    }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     int cid = frontier_take<NS>(fr, lane, far);
+    const bool was_in_group = in_group;
     if (exact && have_tie) {
       const float d = cid >= 0 ? frontier_key_of<NS>(fr, (uint32_t)cid) : INFINITY;
       if (in_group && cid >= 0 && d < group_key) {
@@ -1079,7 +1156,11 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
         }
       }
     }
+    // the trail: over for good, or the hops of a group of equal keys begin or end with the next one
+    if (twin_phase || gave_up || cid < 0) trail_stop(tr, st.n_hops, st.n_dist);
+    else if (in_group != was_in_group) trail_mark(tr, in_group ? kTrailOwn : kTrailBack, st.n_hops + 1, lane);
     if (gave_up || cid < 0) break;
+    hop_cid = cid;
     st.n_hops += 1;
     wave_sync();
     n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
@@ -1101,15 +1182,25 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
 // entered into the filter.
 template <int DT, int QR, int NS>
 __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec<QR>& qv, int ef, Scratch& s, SearchState& st,
-                                                  Frontier<NS>& fr, int n_seed, int lane, bool* ambiguous) {
+                                                  Frontier<NS>& fr, int n_seed, int lane, bool* ambiguous,
+                                                  const uint4* trail = nullptr, int trail_n = 0, int trail_hops = 0,
+                                                  int trail_n_dist = 0) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
   const int S = row_stride(ix, 0);
   int n = n_seed;
   bool amb = false;
+  // The first trail_hops expansions were made by the sorted-set pass too: outside the stretches its markers
+  // set apart, their accepted entries come from its trail (records in hop order, none for a hop that accepted
+  // nothing) instead of from link rows and vectors.  Every entry goes through the accept rule again: it
+  // passes as it did there.
+  int trail_at = 0;
+  bool from_trail = false;
+  bool own_stretch = false;  // between two markers: hops this pass makes itself
+  if (trail_hops > 0) st.n_dist += trail_n_dist;  // the evaluations that pass made up to the trail's end count as performed
   while (true) {
-    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
-    st.n_dist += n;
+    if (n > 0 && !from_trail) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    st.n_dist += from_trail ? 0 : n;
     wave_sync();
     for (int base = 0; base < n; base += 64) {
       const int mine = base + lane;
@@ -1166,7 +1257,43 @@ __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec
     wave_sync();
     if (cid < 0) break;
     st.n_hops += 1;
-    n = visit_lossy(link_row(ix, (uint32_t)cid, 0), S, s, lane);
+    from_trail = false;
+    if (st.n_hops <= trail_hops) {
+      // markers that take effect with this hop (a group may end and the next begin at the same one)
+      while (true) {
+        const uint4 m = trail[trail_at < trail_n ? trail_at : 0];
+        const uint32_t kind = (uint32_t)__builtin_amdgcn_readfirstlane((int)m.x);
+        const uint32_t at_hop = (uint32_t)__builtin_amdgcn_readfirstlane((int)m.w);
+        if (trail_at >= trail_n || kind < kTrailBack || at_hop != (uint32_t)st.n_hops) break;
+        own_stretch = kind == kTrailOwn;
+        trail_at += 1;
+      }
+      if (!own_stretch) {
+        // this hop's records: a run from trail_at on (at most one link row's worth: under 64)
+        const bool have = trail_at + lane < trail_n;
+        const uint4 r = trail[have ? trail_at + lane : 0];
+        const bool mine = have && r.x < kTrailBack && r.w == (uint32_t)st.n_hops;
+        const unsigned long long run = __ballot(mine);
+        const bool wrong = mine && r.x != (uint32_t)cid;
+        if (__ballot(wrong) != 0ull) {
+          trail_hops = 0;  // not the node that pass expanded here: nothing more is taken from the trail
+        } else {
+          n = __popcll(run);
+          if (mine) {
+            s.nbuf[lane] = r.y;
+            s.dbuf[lane] = __uint_as_float(r.z);
+            // (the filter learns the node: a later hop this pass makes itself need not evaluate it again)
+            uint2* sets = reinterpret_cast<uint2*>(s.vcache);
+            const int set_bits = s.vc_bits - 1;
+            const uint32_t slot = r.y & ((1u << set_bits) - 1u);
+            sets[slot] = filter_push(sets[slot], r.y >> set_bits);
+          }
+          trail_at += n;
+          from_trail = true;
+        }
+      }
+    }
+    if (!from_trail) n = visit_lossy(link_row(ix, (uint32_t)cid, 0), S, s, lane);
     wave_sync();
   }
   *ambiguous = amb;

@@ -138,6 +138,7 @@ class Engine {
   int fast_path = 1;     // 0: search with the literal queues only; 1: sorted-set pass first when the batch is
                          // larger than one round of literal wavefronts; 2: always
   int last_repeats = 0;  // queries of the last search that were repeated with the literal queues
+  int last_trails = 0;   // how many of them came with the first pass's trail
   int count_build_work = 0;    // count the work of a build on the device (cuhnsw_last_build_counters)
   unsigned long long build_counters[10] = {};
   int last_build_dropped = 0;  // reverse links of the last build that found no room in an inbox
@@ -162,6 +163,11 @@ class Engine {
   DevBuf<int> d_ctl;  // [0] work counter, [1] status, [2] dirty count, [32] queries given up by the
                       // sorted-set pass, [64] queries it has finished with, [96] work counter of a concurrent literal pass
   DevBuf<int> d_redo;  // their indices
+  DevBuf<uint4> d_trail;      // trails of the sorted-set pass: one buffer per wavefront and the spares,
+  DevBuf<int4> d_redo_trail;  // and which of them goes with which entry of d_redo
+  int trails = 1;             // 0 = the literal pass searches every handed-over query from its entry point
+  int trail_cap = 2048;       // records (accepted entries) per trail; a search that outgrows it leaves none
+  int trail_spares = 1024;    // hand-overs with a trail per batch; the ones after that leave none
   DevBuf<uint4> d_entry;      // longest queries first: level-0 entry of every query of the batch,
   DevBuf<int> d_order_hist;   // bucket counters,
   DevBuf<int> d_order;        // and the order the first pass takes the queries in
@@ -441,7 +447,12 @@ class Engine {
     a.entry = nullptr;
     a.order_hist = nullptr;
     a.order = nullptr;
+    a.trail = nullptr;
+    a.redo_trail = nullptr;
+    a.trail_next = nullptr;
+    a.trail_cap = a.trail_first_spare = a.trail_spares = 0;
     last_repeats = 0;
+    last_trails = 0;
     if (use_static) {
       launch_search_static<DT, QR, NS>(ix, a, ms);
       return;
@@ -543,12 +554,33 @@ class Engine {
       const long long resident = pair ? 2LL * slots : slots;  // queries at work at a time
       // (and up to 32 rounds: what the order saves is part of one round, what the separate descents cost grows
       // with the batch — 1 000 000 queries, 145 rounds: 211.7 against 201.9 ms in the caller's order)
+      // A handed-over query is not searched again from its entry point: the first pass leaves the entries it
+      // accepted, hop by hop, and the literal pass (on the sorted set with ids: it needs no visited bitmap
+      // brought up to date) replays its queue operations from them up to where the two may part.  One query per
+      // wavefront, link rows of one pass of 64 lanes, and batches of up to two rounds of wavefronts: keeping the
+      // trail costs the first pass 2 to 3 %, which only a batch short enough to wait for its last hand-over
+      // gets back (1.18 M x 50, longest first, eight draws of 10 000 queries: 2.75 -> 2.65 ms on average, the
+      // slowest draws 3.06 -> 2.88; 40 000 queries: 6.24 -> 6.39 ms with trails kept).  trails = 2: whatever the batch.
+      const bool keep_trails = (QR == 1 || QR == 2) && trails && !pair && !a.reverse && a.lean && host.S0 <= 63 &&
+                               (trails > 1 || a.nq <= 2 * resident);
+      // (with trails a late hand-over costs less, and the order pays from one round on)
       const bool in_order = query_order && (query_order > 1 ? a.nq > resident
-                                                             : 2 * a.nq >= 3 * resident && a.nq <= 32 * resident);
+                                                             : (keep_trails ? a.nq > resident : 2 * a.nq >= 3 * resident) &&
+                                                                   a.nq <= 32 * resident);
       if (in_order) {
         d_entry.reserve((size_t)a.nq);
         d_order.reserve((size_t)a.nq);
         d_order_hist.reserve((size_t)kOrderBuckets);
+      }
+      if (keep_trails) {
+        d_trail.reserve((size_t)(slots + trail_spares) * trail_cap);
+        d_redo_trail.reserve((size_t)a.nq);
+        a.trail = d_trail.p;
+        a.trail_cap = trail_cap;
+        a.trail_first_spare = slots;
+        a.trail_spares = trail_spares;
+        a.trail_next = d_ctl.p + 48;
+        a.redo_trail = d_redo_trail.p;
       }
       if (side) {
         SearchArgs b = a;
@@ -600,10 +632,11 @@ class Engine {
       if (side) {
         HIP_CHECK(hipStreamWaitEvent(stream, ev_side1, 0));
       }
-      int ctl[33];
+      int ctl[49];
       HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
       HIP_CHECK(hipStreamSynchronize(stream));
       n_literal = last_repeats = ctl[32];
+      last_trails = ctl[48];
       last_repeat_share = (double)n_literal / a.nq;
       share_known = true;
       // an index whose distances tie all the time (integer-valued data) sends most queries
@@ -1157,6 +1190,7 @@ int cuhnsw_enter_point(cuhnsw_engine* e) { return e ? (int)e->impl.host.enterpoi
 int cuhnsw_has_device(void) { return cuhnsw_amd::device_present() ? 1 : 0; }
 double cuhnsw_last_build_seconds(cuhnsw_engine* e) { return e ? e->impl.last_build_seconds : 0.0; }
 int cuhnsw_last_search_repeats(cuhnsw_engine* e) { return e ? e->impl.last_repeats : 0; }
+int cuhnsw_last_search_trails(cuhnsw_engine* e) { return e ? e->impl.last_trails : 0; }
 int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   if (!e || !name) return -1;
   std::string n(name);
@@ -1169,6 +1203,9 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "own_links0") e->impl.own_links0 = (int)value;
   else if (n == "fast_path") e->impl.fast_path = (int)value;
   else if (n == "lean_literal") e->impl.lean_literal = (int)value;
+  else if (n == "trails") e->impl.trails = (int)value;
+  else if (n == "trail_cap") e->impl.trail_cap = std::max(1, (int)value);
+  else if (n == "trail_spares") e->impl.trail_spares = std::max(0, (int)value);
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
   else if (n == "pair_path") e->impl.pair_path = (int)value;
   else if (n == "query_order") e->impl.query_order = (int)value;

@@ -76,6 +76,14 @@ struct SearchArgs {
   uint4* entry;     // per query: level-0 entry point, its key (bits), evaluations and sweeps of the descent
   int* order_hist;  // kOrderBuckets counters, then cursors
   int* order;       // nq query indices, largest entry key first
+  // Trails of the sorted-set pass (device_core.h, struct Trail), all null / 0 = none are kept.  Buffer b holds
+  // trail_cap records from trail + b * trail_cap on; wavefront w of the sorted-set pass starts on buffer w and,
+  // each time it hands over a query whose trail the literal pass is to read, goes on with the next unused one
+  // of the trail_spares buffers behind those (trail_next counts them; none left: it keeps no more trails).
+  uint4* trail;
+  int trail_cap, trail_first_spare, trail_spares;
+  int* trail_next;
+  int4* redo_trail;  // per entry of a.redo: (buffer or -1, records, expansions covered, evaluations up to there)
 };
 
 struct BuildArgs {
@@ -376,6 +384,9 @@ __global__ void __launch_bounds__(1024) order_scatter_kernel(const uint4* entry,
 // held to 72 registers, seven wavefronts per SIMD, at the price of up to five spilled registers;
 // eight wavefronts are no faster; with eight keys per lane it fits 96 registers, five wavefronts
 // per SIMD, without spilling; the other shapes would spill heavily)
+// With a.trail set the pass leaves trails for the literal pass (2 to 3 % more instructions: the host asks for
+// them in batches of a round or two of wavefronts, where a query handed over late is a good part of the
+// batch's time).
 template <int DT, int QR, int NS>
 __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS == 8 ? 5 : 1)) : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -389,6 +400,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
   s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
   // tells a literal pass waiting beside this one that the two kernels do run at the same time
   if (blockIdx.x == 0 && lane == 0) __hip_atomic_store(a.done + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  int trail_buf = a.trail ? (int)blockIdx.x : -1;  // the buffer this wavefront's trails go to
 
   for (;;) {
     int qi = 0;
@@ -398,6 +410,12 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     }
     qi = __builtin_amdgcn_readfirstlane(qi);
     if (qi >= a.nq) break;
+    Trail tr;
+    if (trail_buf >= 0) {
+      tr.rec = a.trail + (size_t)trail_buf * a.trail_cap;
+      tr.cap = a.trail_cap;
+      tr.on = true;
+    }
     QVec<QR> qv;
     load_query<QR>(qv, s.qlds, a.q + (size_t)qi * ix.D, ix.D, ix.Dp, lane);
     SearchState st;
@@ -423,7 +441,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     wave_sync();
     // (the flag is made wavefront-uniform explicitly and both outcomes are plain branches)
     const int how =
-        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0, a.k >= a.ef));
+        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0, a.k >= a.ef, &tr));
     const int T0 = st.top_size < a.k ? st.top_size : a.k;
     // Equal keys across the cut at k: which of them stays is up to the result heap, which the
     // literal search reproduces.  Equal keys among the k best: the answer lists them by label.
@@ -432,9 +450,20 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
         (how == 2 && !a.reverse && frontier_tie_within<NS>(fr, a.ef, T0 - 1, st.top_size, lane)) ? 1 : 0);
     const bool gave_up = how == 1 || cut_tie || (inner_tie && T0 > (1 << a.fc_bits));  // (the filter's LDS is the sort's buffer)
     if (gave_up) {
+      // (the trail's records are written by many lanes: all of them out before lane 0 publishes the entry)
+      const bool with_trail = a.redo_trail && trail_buf >= 0 && tr.n > 0 && tr.hops > 0;
+      if (with_trail) __threadfence();
+      int spare = 0;
       if (lane == 0) {
         const int slot = atomicAdd(a.repeats, 1);
+        if (a.redo_trail) a.redo_trail[slot] = make_int4(with_trail ? trail_buf : -1, tr.n, tr.hops, tr.n_dist);
         __hip_atomic_store(&a.redo[slot], qi, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        if (with_trail) spare = atomicAdd(a.trail_next, 1);
+      }
+      if (with_trail) {
+        // that buffer belongs to the literal pass now
+        spare = __builtin_amdgcn_readfirstlane(spare);
+        trail_buf = spare < a.trail_spares ? a.trail_first_spare + spare : -1;
       }
     } else {
       const int T = __builtin_amdgcn_readfirstlane(st.top_size < a.k ? st.top_size : a.k);
@@ -852,9 +881,11 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
 
   for (;;) {
     int qi = 0;
+    int entry = 0;  // which entry of the list this is
     if (lane == 0) {
       qi = atomicAdd(a.counter, 1);
       if (a.live) {
+        entry = qi;
         // entry qi of the list appears once the sorted-set pass has given up that many
         // queries; it never will if that pass has finished them all and the entry is still
         // empty.  The wait is bounded in wall-clock time: if the first pass has not even started
@@ -909,11 +940,22 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
       } else if (qi >= (a.nq_dev ? *a.nq_dev : a.nq)) {
         qi = -1;
       } else if (a.redo) {
+        entry = qi;
         qi = a.redo[qi];  // second pass: only the queries the sorted-set pass gave up
       }
     }
     qi = __builtin_amdgcn_readfirstlane(qi);
     if (qi < 0) break;
+    // the trail the sorted-set pass left for this query, if any (its records were written by another
+    // wavefront before the list entry was: read them from memory, not from this CU's cache)
+    int4 tmeta = make_int4(-1, 0, 0, 0);
+    if (lean && a.redo_trail) {
+      entry = __builtin_amdgcn_readfirstlane(entry);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      const int4 m = a.redo_trail[entry];
+      tmeta = make_int4(__builtin_amdgcn_readfirstlane(m.x), __builtin_amdgcn_readfirstlane(m.y),
+                        __builtin_amdgcn_readfirstlane(m.z), __builtin_amdgcn_readfirstlane(m.w));
+    }
     // beside the first pass a literal wavefront is one among a few dozen on its CU and its query
     // is on the batch's critical path: it goes first whenever it has an instruction ready
     if (a.live) __builtin_amdgcn_s_setprio(3);
@@ -940,7 +982,9 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
       if (lane == 0) s.nbuf[0] = cur;
       wave_sync();
       bool ambiguous = false;
-      search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous);
+      search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous,
+                                    tmeta.x >= 0 ? a.trail + (size_t)tmeta.x * a.trail_cap : nullptr, tmeta.y,
+                                    tmeta.x >= 0 ? tmeta.z : 0, tmeta.w);
       T = st.top_size < a.k ? st.top_size : a.k;
       // The first T entries of the set (equal keys among them in label order) are hnswlib's
       // answer unless equal keys sit across the cut, or the whole set is returned after an

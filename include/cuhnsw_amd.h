@@ -144,6 +144,11 @@ int cuhnsw_debug_link_keys0(cuhnsw_engine* e, float* out, long long capacity);
  * by distance alone, which is exact only without ties; the reference has no such distinction
  * because its kernel does not reproduce hnswlib's tie order) */
 int cuhnsw_last_search_repeats(cuhnsw_engine* e);
+/* how many of those queries the literal pass did not search from the entry point again: the first pass had
+ * left the entries it accepted, hop by hop (its trail), and the literal pass replayed its queue operations
+ * from them up to the point where the two searches may part (tunable "trails"; no counterpart in the
+ * reference) */
+int cuhnsw_last_search_trails(cuhnsw_engine* e);
 /* tuning knobs that are not part of the reference's option table:
  *   "build_batch"   largest number of nodes inserted per batch (default 0 = by the size of the graph: a quarter
  *                   of the nodes already in, at most 16384; beyond 524288 nodes a thirty-second, at most 65536)
@@ -161,7 +166,8 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *                   batch exceeds one round of resident wavefronts, literal queues for the queries
  *                   that met equal distances (default); 2 = first pass whatever the batch size
  *   "filter_entries" entries of the first pass's LDS visited filter (0 = automatic)
- *   "query_order"   1 (default) = a search batch of 1.5 to 32 rounds of wavefronts does its upper-level descents
+ *   "query_order"   1 (default) = a search batch of 1.5 to 32 rounds of wavefronts (from one round on where the
+ *                   first pass keeps trails) does its upper-level descents
  *                   first and takes its queries by descending distance of their level-0 entry point (the longest
  *                   searches first: a launch ends when its last query does); 2 = from more than one round on;
  *                   0 = in the caller's order.  Same answers and counters either way.
@@ -184,6 +190,16 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  *   "lean_literal"  visited set of the literal-queue pass: 0 = exact bitmap in HBM (one bit per point and
  *                   wavefront), 2 = tag filter in LDS with the sorted set catching repeats, 1 = automatic
  *                   (the bitmap while all bitmaps at work fit the L2 caches; default)
+ *   "trails"        1 = the first pass leaves, per query, the entries it accepted hop by hop while its course is
+ *                   certainly hnswlib's; the literal pass starts a handed-over query from there instead of from
+ *                   the entry point (cuhnsw_last_search_trails counts them).  Needs the literal pass on the tag
+ *                   filter (lean_literal), one query per wavefront, link rows under 64 ids, vectors of up to
+ *                   128 elements; 266 MB of device memory for 2048 accepted entries per query at work.  Keeping
+ *                   the trail costs the first pass 2 to 3 %: 1 (default) = for batches of up to two rounds of
+ *                   wavefronts, which wait for their last hand-over; 2 = for every batch; 0 = off.
+ *   "trail_cap"     accepted entries a trail holds (default 2048; a search that accepts more leaves none)
+ *   "trail_spares"  handed-over queries per batch that can come with a trail (default 1024: each keeps the
+ *                   buffer it was written to until the batch is over; the ones after that come without)
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)

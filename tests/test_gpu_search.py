@@ -324,6 +324,54 @@ def test_literal_pass_schedules_on_tie_heavy_data(oracle, tmp_path):
     _check_parity(oracle, ix, e, q, 100, 100)
 
 
+@pytest.mark.parametrize("d,hi", [(16, 30), (12, 60), (80, 6)], ids=["many_ties", "fewer_ties", "two_chunks_per_lane"])
+def test_handed_over_queries_start_from_the_first_pass_trail(oracle, tmp_path, d, hi):
+  """The first pass leaves the entries it accepted, hop by hop, and the literal pass (on the tag filter) replays
+  its queue operations from them instead of searching a handed-over query from the entry point: same answers and
+  hop counters as the oracle — with a trail for every handed-over query, for a few only (no spare buffers after
+  three), with trails that overflow (16 entries), and with none."""
+  n = 5000
+  x = integer_vectors(n, d, seed=61, hi=hi)
+  q = integer_vectors(250, d, seed=62, hi=hi)   # (under 256 queries: the engine keeps trying the first pass however many tie)
+  mult = 1 / np.log(8)
+  ix = oracle.OracleIndex("l2").build(x, _levels(n, mult, 63), 8, 16, 60, mult)
+  p = str(tmp_path / "t.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
+  e.load_index(p)
+  e.set_tunable("fast_path", 2)
+  e.set_tunable("lean_literal", 2)
+  e.set_tunable("pair_path", 0)
+  for k, ef in ((10, 100), (100, 100), (10, 300)):
+    o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
+    # (eight wavefronts: each answers some thirty queries and needs a spare buffer after every hand-over; trails = 2:
+    # also in a batch of many rounds of wavefronts)
+    for name, settings in (("all", {}), ("eight", {"search_slots": 8, "trails": 2}), ("three", {"search_slots": 8, "trails": 2, "trail_spares": 3}),
+                           ("short", {"trail_cap": 16}), ("after", {"concurrent_literal": 0}), ("none", {"trails": 0})):
+      for key, value in {"trails": 1, "trail_cap": 2048, "trail_spares": 1024, "concurrent_literal": 1, "search_slots": 0,
+                         **settings}.items():
+        e.set_tunable(key, value)
+      g_ids, g_d, g_f, stats = _device_search(e, q, k, ef)
+      assert (g_f == o_f).all()
+      for r in range(q.shape[0]):
+        f = o_f[r]
+        assert (g_ids[r, :f] == o_ids[r, :f]).all() and (g_d[r, :f] == o_d[r, :f]).all(), (name, k, ef, r)
+      assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
+      handed, trails = e.last_search_repeats, e.last_search_trails
+      assert handed > 0, (name, k, ef, handed, trails)
+      if name in ("all", "after", "eight"):
+        assert trails == handed
+      elif name == "three":
+        assert trails <= 8 + 3 and (trails < handed or handed <= 11)   # the wavefronts' own buffers and the spares
+      elif name == "short":
+        assert trails <= handed
+      else:
+        assert trails == 0
+  for key, value in (("trails", 1), ("trail_cap", 2048), ("trail_spares", 1024), ("concurrent_literal", 1), ("pair_path", 1),
+                     ("search_slots", 0)):
+    e.set_tunable(key, value)
+
+
 def test_overflowing_scratch_areas_are_retried(oracle, tmp_path):
   """Accept log and queue overflow area start far too small: the engine must notice, grow
   them and repeat the search with unchanged answers."""
