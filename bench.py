@@ -125,7 +125,7 @@ def main():
   ap.add_argument("--fast-path", type=int, default=1, choices=[0, 1, 2],
                   help="0 = literal priority queues only, 1 = default, 2 = sorted-set first pass whatever the batch size")
   ap.add_argument("--pair-path", type=int, default=1, choices=[0, 1, 2],
-                  help="0 = never two queries per wavefront in the first pass, 2 = wherever the shapes allow it")
+                  help="2 = two queries per wavefront in the first pass wherever the shapes allow it, 0 = never, 1 = the engine's choice (at present: never)")
   ap.add_argument("--query-order", type=int, default=1, choices=[0, 1, 2],
                   help="0 = queries in the caller's order, 1 = longest first from one to one and a half rounds of wavefronts on, 2 = from one")
   ap.add_argument("--trails", type=int, default=1, choices=[0, 1, 2],
@@ -326,7 +326,7 @@ def main():
                     "queries_repeated_with_literal_queues": int(repeats)},
       "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                    "frac": achieved / 8000.0, "traffic": traffic,
-                   "kernel": ("search_pair_kernel" if (args.pair_path and d <= 128 and (ef <= 64 or (ef <= 128 and nq >= 14336))) else "search_fast_kernel") +
+                   "kernel": ("search_pair_kernel" if (args.pair_path == 2 and d <= 128 and ef <= 128) else "search_fast_kernel") +
                              " with search_kernel beside it (one search of the batch)"
                              if args.fast_path else "search_kernel (literal priority queues only)",
                    "algorithmic_bytes_per_launch": gather_bytes},

@@ -129,7 +129,7 @@ class Engine {
   int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   int first_pass_waves = 0;  // wavefronts per CU of the first pass (0 = as many as fit)
-  int pair_path = 1;       // first pass with two queries per wavefront where the shapes allow it (0: one per wavefront)
+  int pair_path = 1;       // first pass with two queries per wavefront: 2 = where the shapes allow it, 0 / 1 = never (1: automatic)
   int query_order = 1;     // first pass of 1.5 to 32 rounds of wavefronts: longest queries first (0: caller's order)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
@@ -500,14 +500,13 @@ class Engine {
       constexpr bool kPairShape = (QR == 1 || QR == 2) && NS == 2;
       constexpr int N2 = kPairShape ? 2 * NS : 2;
       auto pair_kernel = search_pair_kernel<DT, (kPairShape ? QR : 1), N2>;
-      // (measured: at ef_search up to 64 the pair kernel is the faster one whatever the batch; between 65 and 128
-      // it wins once the batch is several rounds of wavefronts — 1.18 M x 50, 40 000 queries, ef 128: 5.5 against
-      // 6.5 ms; 10 M x 96, 100 000 queries: 20.0 against 21.3 ms — and loses where the whole batch is resident at
-      // once and a query's own latency is what counts — 1 M x 128, 10 000 queries, ef 128: 2.95 against 2.68 ms;
-      // pair_path = 2 forces it)
-      const int single_slots = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits).total);
-      const bool pair = kPairShape && pair_path != 0 && !a.reverse && host.S0 <= 32 && host.SU <= 32 && a.nq > 1 &&
-                        (pair_path > 1 || a.ef <= 64 || a.nq >= 2 * single_slots);
+      // (pair_path = 2 asks for it.  It used to be the faster kernel at ef_search up to 64, and up to 128 on batches
+      // of several rounds of wavefronts — 1.18 M x 50, 40 000 queries, ef 128: 5.5 against 6.5 ms.  Against the
+      // one-query kernel as it is built now it no longer is, anywhere measured: 1.18 M x 50, 40 000 queries, ef 32 /
+      // 64 / 128: 2.68 / 3.20 / 4.40 ms against 2.70 / 3.08 / 3.99; 10 M x 96, 100 000 queries, ef 64 / 128: 16.4 /
+      // 18.5 against 14.1 / 15.4 ms; 1 M x 128, 10 000 queries, ef 64: 2.10 against 1.62 ms.  So the automatic
+      // setting, pair_path = 1, does not choose it at present.)
+      const bool pair = kPairShape && pair_path > 1 && !a.reverse && host.S0 <= 32 && host.SU <= 32 && a.nq > 1;
       auto fast_lds = [&](int bits) -> size_t {
         return pair ? plan_pair_lds(a.lcap, bits).total : plan_fast_lds(QR, ix.Dp, a.lcap, bits).total;
       };

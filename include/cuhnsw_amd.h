@@ -171,10 +171,10 @@ int cuhnsw_last_search_trails(cuhnsw_engine* e);
  *                   first and takes its queries by descending distance of their level-0 entry point (the longest
  *                   searches first: a launch ends when its last query does); 2 = from more than one round on;
  *                   0 = in the caller's order.  Same answers and counters either way.
- *   "pair_path"     1 = the first pass runs two queries per wavefront (32 lanes each) where that is the faster
- *                   shape: ef_search up to 64, or up to 128 with a batch of several rounds of wavefronts; vectors
- *                   of at most 128 dimensions, max_m and max_m0 at most 32 (default); 2 = wherever the shapes
- *                   allow it (ef_search up to 128); 0 = always one query per wavefront.  Same results either way.
+ *   "pair_path"     2 = the first pass runs two queries per wavefront (32 lanes each) wherever the shapes allow
+ *                   it: ef_search up to 128, vectors of at most 128 dimensions, max_m and max_m0 at most 32;
+ *                   0 = always one query per wavefront; 1 (default) = whichever is the faster one, which at
+ *                   present is one query per wavefront in every measured shape.  Same results either way.
  *   "first_pass_waves" wavefronts per CU of the first pass (0 = as many as fit, the default)
  *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
  *                   (default), 0 = after it
