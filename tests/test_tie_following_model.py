@@ -5,15 +5,33 @@ the time, and whenever it does NOT give a query up, its answer — ids, distance
 of expansions and evaluations — must be what the oracle's literal hnswlib search
 (two std::priority_queues) returns.  A rule that lets an order-dependent case through shows
 up here as a mismatch within a few thousand trials.  (The rules include the one that follows the two
-twins of an eviction out of two equal largest keys through instead of giving the query up.)"""
+twins of an eviction out of two equal largest keys through instead of giving the query up.)
+
+The same model also keeps the TRAIL the first pass leaves for the literal pass (struct Trail in device_core.h): the
+entries accepted hop by hop, no records but two markers around the hops of a group of equal keys, nothing after the
+twins of an eviction come up.  A second model, hnswlib's search on literal libstdc++ heaps, replays a given-up
+query from that trail — recorded hops take their accepted entries from the records and evaluate nothing, the
+others are made for real — and must arrive at the oracle's answer and hop count: what a hop accepts does not depend
+on the order in which a followed-through group was expanded, which is what the replay on the GPU rests on."""
 import numpy as np
 import pytest
 
 INF = float("inf")
 
 
-def sorted_set_search(keys_of, rows, ep, k, ef):
-  """Returns None when given up, else (ids, keys, hops, evaluations, met equal keys)."""
+def sorted_set_search(keys_of, rows, ep, k, ef, trail=None):
+  """Returns None when given up, else (ids, keys, hops, evaluations, met equal keys).  trail: a dict that receives
+  "rec" (the records and markers) and "hops" (the expansions they cover)."""
+  tr = {"rec": [], "on": True, "own": False, "hops": 0}
+
+  def stop(h):                            # the trail ends: h expansions are complete
+    if tr["on"]:
+      tr["on"] = False
+      tr["hops"] = h
+    if trail is not None:
+      trail["rec"], trail["hops"] = tr["rec"], tr["hops"]
+
+  hop_node = None                         # the node the current hop expanded (None: the seed)
   S = [[keys_of(ep), ep, False]]          # sorted by key, equal keys in order of arrival
   seen = {ep}
   have_tie = in_group = False
@@ -26,6 +44,7 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
   hops = 0
   offers = []
   while True:
+    accepted = []
     for key, node in offers:
       full = len(S) >= ef
       if full and not (S[-1][0] > key):
@@ -40,10 +59,12 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
       while pos > 0 and S[pos - 1][0] > key:
         pos -= 1
       S.insert(pos, [key, node, False])
+      accepted.append((key, node))
       if len(S) > ef:
         if in_group:
           group_edge = min(group_edge, S[-1][0])
           if S[-1][0] == group_key and not S[-1][2]:
+            stop(hops - 1)
             return None                       # a member of the group pushed out before its turn
         S.pop()
       if twins:
@@ -52,22 +73,29 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
         # three equal largest keys, a second such eviction, or the whole set asked for: the plain rule
         ghosts += 2 if (S[-1][0] == S[-2][0] or k >= ef) else 1
       if twin_phase:
+        stop(hops - 1)
         return None                           # which twin goes first now decides whether the other is expanded at all
+    if tr["on"] and not tr["own"] and hop_node is not None:
+      tr["rec"] += [("rec", hop_node, node, key, hops) for key, node in accepted]
+    was_in_group = in_group
     pick = next((i for i, e in enumerate(S) if not e[2]), -1)
     d = S[pick][0] if pick >= 0 else INF
     if in_group and pick >= 0 and d < group_key:
       # a closer candidate turned up inside the group: it is expanded before the rest of the group under
       # any order; a group within the group is not followed
       if any((not e[2]) and e[0] == d for i, e in enumerate(S) if i != pick):
+        stop(hops)
         return None
     elif in_group and d != group_key:
       # the group is through: with another order of its members an offer or an entry whose key
       # equals the bound reached now could have ended up on the other side of it, and with the bound
       # below the group's key a member popped late would not have been expanded at all
       if len(S) >= ef and (group_edge == S[-1][0] or S[-1][0] < group_key):
+        stop(hops)
         return None
       in_group = False
     if pick < 0:
+      stop(hops)
       if len(S) >= ef and S[-1][0] >= ek_min:
         # an evicted twin is still a live candidate of hnswlib
         if ghosts != 1:
@@ -90,11 +118,18 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
         if ghosts == 1 and not in_group and not others:
           twin_phase = True
         else:
+          stop(hops)
           return None
       if not in_group and not twin_phase:
         in_group = any((not e[2]) and e[0] == d for i, e in enumerate(S) if i != pick)
         group_key = d
         group_edge = INF
+    if twin_phase:
+      stop(hops)
+    elif tr["on"] and in_group != was_in_group:
+      tr["rec"].append(("own" if in_group else "back", hops + 1))
+      tr["own"] = in_group
+    hop_node = S[pick][1]
     S[pick][2] = True
     hops += 1
     offers = []
@@ -104,13 +139,161 @@ def sorted_set_search(keys_of, rows, ep, k, ef):
         offers.append((keys_of(nb), nb))
   T = min(k, len(S))
   if have_tie and T < len(S) and S[T - 1][0] == S[T][0]:
-    return None                               # equal keys across the cut: the result heap's choice
+    return None                               # equal keys across the cut: the result heap's choice (the trail is complete)
   best = sorted((e[0], e[1]) for e in S[:T])  # equal keys among the k best: listed by label
   sorted_set_search.answered_after_twins += bool(twin_phase)
   return [e[1] for e in best], [e[0] for e in best], hops, len(seen), have_tie
 
 
 sorted_set_search.answered_after_twins = 0    # (statistics for the test below: the twin rule has to be exercised)
+
+
+def _push_heap(h, value):
+  """std::push_heap after push_back, max-heap on value[0] (bits/stl_heap.h, __push_heap)."""
+  h.append(value)
+  hole = len(h) - 1
+  while hole > 0:
+    parent = (hole - 1) // 2
+    if not (h[parent][0] < value[0]):
+      break
+    h[hole] = h[parent]
+    hole = parent
+  h[hole] = value
+
+
+def _pop_heap(h):
+  """std::pop_heap + pop_back (bits/stl_heap.h, __pop_heap / __adjust_heap); returns the former top."""
+  top = h[0]
+  value = h.pop()
+  n = len(h)
+  if n == 0:
+    return top
+  hole = child = 0
+  while child < (n - 1) // 2:
+    child = 2 * (child + 1)
+    if h[child][0] < h[child - 1][0]:
+      child -= 1
+    h[hole] = h[child]
+    hole = child
+  if n % 2 == 0 and child == (n - 2) // 2:
+    child = 2 * (child + 1)
+    h[hole] = h[child - 1]
+    hole = child - 1
+  while hole > 0:                             # __push_heap(first, hole, 0, value)
+    parent = (hole - 1) // 2
+    if not (h[parent][0] < value[0]):
+      break
+    h[hole] = h[parent]
+    hole = parent
+  h[hole] = value
+  return top
+
+
+def literal_search(keys_of, rows, ep, k, ef, trail=None):
+  """hnswlib's searchBaseLayerST + searchKnn on two literal priority queues (hnswalg.h).  With a trail: the
+  expansions it covers take their accepted entries from its records and evaluate nothing (their neighbours only
+  become visited), except inside the stretches its markers set apart, which are made for real.
+  Returns (ids, keys, hops, evaluations made)."""
+  rec = trail["rec"] if trail else []
+  covered = trail["hops"] if trail else 0
+  at = 0
+  own = False
+  top, cand = [], []                          # (key, id) max-heap; (-key, id) max-heap
+  d0 = keys_of(ep)
+  _push_heap(top, (d0, ep))
+  _push_heap(cand, (-d0, ep))
+  lower = d0
+  visited = {ep}
+  hops = evals = 0
+  while cand:
+    if -cand[0][0] > lower:
+      break
+    node = _pop_heap(cand)[1]
+    hops += 1
+    offers = None
+    if hops <= covered:
+      while at < len(rec) and rec[at][0] != "rec" and rec[at][1] == hops:
+        own = rec[at][0] == "own"
+        at += 1
+      if not own:
+        offers = []
+        while at < len(rec) and rec[at][0] == "rec" and rec[at][4] == hops:
+          assert rec[at][1] == node, "the trail names another node for this hop"
+          offers.append((rec[at][3], rec[at][2]))
+          at += 1
+        visited.update(rows[node])
+    if offers is None:
+      offers = []
+      for nb in rows[node]:
+        if nb not in visited:
+          visited.add(nb)
+          evals += 1
+          offers.append((keys_of(nb), nb))
+    for key, nb in offers:
+      if len(top) < ef or lower > key:
+        if hops <= covered and not own:
+          pass                                # (a recorded entry: it passes, as it did in the first pass)
+        _push_heap(cand, (-key, nb))
+        _push_heap(top, (key, nb))
+        if len(top) > ef:
+          _pop_heap(top)
+        lower = top[0][0]
+      else:
+        assert not (hops <= covered and not own), "a recorded entry is turned away"
+  while len(top) > k:
+    _pop_heap(top)
+  best = sorted(top)
+  return [e[1] for e in best], [e[0] for e in best], hops, evals
+
+
+@pytest.mark.parametrize("seed", list(range(4)))
+def test_given_up_queries_replayed_from_the_trail_match_the_oracle(oracle, seed):
+  rng = np.random.default_rng(5000 + seed)
+  replayed = with_markers = covered_hops = all_hops = plain = 0
+  for graph in range(60):
+    n = int(rng.integers(12, 60))
+    dim = int(rng.integers(1, 4))
+    hi = int(rng.integers(3, 30))
+    x = rng.integers(0, hi, (n, dim)).astype(np.float32)
+    deg = int(rng.integers(2, 7))
+    links0 = np.zeros((n, 1 + 8), np.uint32)
+    rows = []
+    for i in range(n):
+      others = [j for j in range(n) if j != i]
+      nb = list(rng.choice(others, size=min(deg, len(others)), replace=False))
+      nb.append((i + 1) % n)
+      nb = list(dict.fromkeys(int(v) for v in nb if v != i))[:8]
+      links0[i, 0] = len(nb)
+      links0[i, 1:1 + len(nb)] = nb
+      rows.append(nb)
+    ix = oracle.OracleIndex("l2").from_arrays(x, np.zeros(n, np.int32), links0, np.zeros(0, np.uint32),
+                                              max_m=4, max_m0=8, maxlevel=0, enterpoint=0)
+    q = rng.integers(0, hi, (24, dim)).astype(np.float32)
+    for k, ef in ((1, 1), (2, 3), (3, 5), (4, 4), (5, 8), (2, 12)):
+      ids, dists, found, cnt = ix.search(q, k, ef, convention="hnswlib", counters=True)
+      for r in range(q.shape[0]):
+        keys_of = lambda node, qq=q[r]: float(np.float32(((qq - x[node]) ** 2).sum()))
+        f = found[r]
+        if r < 2:
+          # the literal model by itself is the oracle's search (this pins the Python heaps)
+          l_ids, l_keys, l_hops, l_evals = literal_search(keys_of, rows, 0, k, ef)
+          assert l_ids == list(ids[r, :f]) and l_keys == list(dists[r, :f]) and l_hops == cnt[r, 1]
+          assert l_evals + 1 == cnt[r, 0]
+          plain += 1
+        trail = {}
+        if sorted_set_search(keys_of, rows, 0, k, ef, trail) is not None or not trail.get("rec") or trail["hops"] == 0:
+          continue
+        l_ids, l_keys, l_hops, l_evals = literal_search(keys_of, rows, 0, k, ef, trail)
+        assert l_ids == list(ids[r, :f]) and l_keys == list(dists[r, :f]), (seed, graph, r, k, ef)
+        assert l_hops == cnt[r, 1], (seed, graph, r, k, ef)
+        replayed += 1
+        with_markers += any(e[0] != "rec" for e in trail["rec"])
+        covered_hops += trail["hops"]
+        all_hops += l_hops
+  # given-up queries with a trail are common on this data, many of their trails lead through a group of equal
+  # keys, and the trails cover a good part of the expansions
+  assert replayed > 1000 and with_markers > 500 and plain > 500, (replayed, with_markers, plain)
+  assert covered_hops * 4 > all_hops, (covered_hops, all_hops)
 
 
 @pytest.mark.parametrize("seed", list(range(6)) + [141])   # 141: the case that showed the need for the rule on the group's edge
