@@ -252,6 +252,7 @@ def main():
     eng.set_tunable("fast_path", args.fast_path)
     step(with_stats=True)
   repeats = eng.last_search_repeats
+  from_trails = eng.last_search_trails
   for _ in range(args.warmup):
     step()
   torch.cuda.synchronize()
@@ -323,7 +324,8 @@ def main():
       "per_query": {"n_dist": float(st[:, 0].mean()), "n_hops": float(st[:, 1].mean()),
                     "n_dist_upper": float(st[:, 2].mean()), "n_sweeps_upper": float(st[:, 3].mean()),
                     "n_dist_performed": float(st_run[:, 0].mean()),
-                    "queries_repeated_with_literal_queues": int(repeats)},
+                    "queries_repeated_with_literal_queues": int(repeats),
+                    "of_them_replayed_from_the_first_pass_trail": int(from_trails)},
       "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                    "frac": achieved / 8000.0, "traffic": traffic,
                    "kernel": ("search_pair_kernel" if (args.pair_path == 2 and d <= 128 and ef <= 128) else "search_fast_kernel") +
