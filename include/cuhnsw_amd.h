@@ -79,7 +79,8 @@ int cuhnsw_search_knn(cuhnsw_engine* e, const float* qdata, int num_queries, int
  * is copied.  Counterpart of the kernel launch inside CuHNSW::SearchGraph
  * (cpp/src/cuhnsw_build.cu:254-275).  d_stats may be null, else int32
  * [num_queries x 4]: level-0 distance evaluations (performed ones: the first pass may evaluate a
- * node again after its visited filter has forgotten it; exact with tunable fast_path = 0), level-0
+ * node again after its visited filter has forgotten it, and for a query answered from a trail the figure is
+ * the first pass's count at the trail's end plus the literal pass's own; exact with tunable fast_path = 0), level-0
  * expanded candidates, upper-level distance evaluations, upper-level sweeps.  The call returns after
  * the kernel has finished; kernel_ms (may be null) receives the kernel's duration
  * measured with HIP events on the engine's stream. */
