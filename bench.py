@@ -298,6 +298,22 @@ def main():
     large = {"queries": nl, "search_ms": float(np.mean(l_ms)), "value": nl / (float(np.mean(l_ms)) * 1e-3), "unit": "queries/s"}
     del ql, l_nns, l_dist, l_found
 
+  # The batch's time depends on whether, and when, one of its queries is handed to the literal pass: eight other
+  # draws of as many queries from the same law (not part of `value`, which is quoted on the configuration's own queries).
+  other_draws = None
+  if args.workload == "C2" and args.n is None and args.nq is None and not args.no_large:
+    times, handed = [], []
+    for draw in range(8):
+      qd = torch.from_numpy(datasets.more_queries(args.workload, nq, draw)).cuda()
+      torch.cuda.synchronize()
+      ms = [eng.search_knn_device(qd.data_ptr(), nq, k, ef, nns.data_ptr(), dist.data_ptr(), found.data_ptr(), None)
+            for _ in range(5)][1:]
+      times.append(float(np.mean(ms)))
+      handed.append(int(eng.last_search_repeats))
+    other_draws = {"draws": len(times), "queries": nq, "mean_ms": float(np.mean(times)), "min_ms": float(min(times)),
+                   "max_ms": float(max(times)), "ms": [round(t, 3) for t in times],
+                   "queries_repeated_with_literal_queues": handed}
+
   avg_kernel_ms = float(np.mean(kernel_ms))
   row_bytes_stored = (2 if args.storage == "fp16" else 4) * d
   gather_bytes = int(st[:, 0].sum()) * (2 if args.storage == "fp16" else 4) * d
@@ -353,6 +369,8 @@ def main():
 
   if large:
     out["large_batch"] = large
+  if other_draws:
+    out["other_draws_of_the_queries"] = other_draws
 
   # the memory system alone: random gathers of this index's rows, with as many wavefronts per CU as the first
   # pass holds and as many rows in flight per wavefront as a hop fetches on average (4) and at most (16)

@@ -85,6 +85,17 @@ def make(name, n=None, nq=None):
   return data, queries, spec
 
 
+def more_queries(name, nq, draw):
+  """Another draw of nq queries from the law of a named config's own queries (draw = 0, 1, ...: the seed)."""
+  spec = CONFIGS[name]
+  qrng = np.random.default_rng(9000 + draw)
+  if spec.get("query_law") == "unit_normal":
+    queries = qrng.standard_normal((nq, spec["d"])).astype(np.float32)
+    return queries / np.linalg.norm(queries, axis=1, keepdims=True)
+  centres = _centres(np.random.default_rng(1000 + spec["cfg"]), spec["law"], spec["centres"], spec["d"])
+  return _draw(qrng, centres, spec["law"], nq)
+
+
 def random_levels(n, level_mult, seed=777):
   """Level stream of the Python wrapper (cuhnsw/pyhnsw.py:65-71 in the
   reference): legacy MT19937 uniform draws, truncated -ln(u) * mult."""
