@@ -3,6 +3,7 @@ and the pybind11 module cuhnsw_bind that wraps it.
 
   python -m cuhnsw_amd.build
 """
+import json
 import os
 import subprocess
 import sys
@@ -24,14 +25,47 @@ HIP_FLAGS = [
 ]
 
 
+RESOURCES = os.path.join(HERE, "..", "profiles", "kernel_resources.json")
+
+
 def _run(cmd):
   print("+", " ".join(cmd), flush=True)
   subprocess.check_call(cmd)
 
 
+def _demangle(names):
+  try:
+    out = subprocess.run(["c++filt"] + names, capture_output=True, text=True, check=True).stdout.split("\n")
+    return [o.strip() for o in out[:len(names)]]
+  except (OSError, subprocess.CalledProcessError):
+    return names
+
+
 def build_lib():
+  """Compiles the library and records, from the compiler's resource-usage remarks of this very build, what
+  every kernel in it takes: registers, spills, scratch bytes, wavefronts per SIMD (profiles/kernel_resources.json;
+  `python -m cuhnsw_amd.kernel_report` adds where in the first-pass kernels the scratch accesses sit)."""
+  from cuhnsw_amd import kernel_report
   srcs = [os.path.join(CSRC, "engine.hip"), os.path.join(CSRC, "index_file.cpp")]
-  _run([HIPCC] + HIP_FLAGS + ["-x", "hip"] + srcs + ["-o", LIB])
+  cmd = [HIPCC] + HIP_FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-x", "hip"] + srcs + ["-o", LIB]
+  print("+", " ".join(cmd), flush=True)
+  r = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+  other = [l for l in r.stderr.split("\n") if "kernel-resource-usage" not in l and "not a recognized feature" not in l
+           and not l.lstrip().startswith(("|", "^", "In file included from")) and "__launch_bounds__" not in l
+           and "__global__" not in l]
+  if "".join(other).strip():
+    print("\n".join(l for l in other if l.strip()), file=sys.stderr)
+  if r.returncode != 0:
+    raise subprocess.CalledProcessError(r.returncode, cmd)
+  usage = kernel_report.parse_remarks(r.stderr)
+  names = sorted(usage)
+  table = {plain: usage[mangled] for mangled, plain in zip(names, _demangle(names))}
+  try:
+    with open(RESOURCES, "w") as f:
+      json.dump({"flags": HIP_FLAGS, "kernels": table}, f, indent=1, sort_keys=True)
+      f.write("\n")
+  except OSError as e:   # a read-only tree: the library is what matters
+    print("kernel resources not recorded:", e, file=sys.stderr)
   return LIB
 
 
