@@ -34,7 +34,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-KERNEL_SOURCES = ["device_core.h", "heap_coop.h", "kernels.h", "pair_search.h", "engine.hip"]
+KERNEL_SOURCES = ["device_core.h", "heap_coop.h", "kernels.h", "engine.hip"]
 
 
 def kernel_source_digest():
@@ -62,7 +62,7 @@ def ingest_pmc(fetch_dir, write_dir, workload):
       name, value = row["Kernel_Name"], float(row["Counter_Value"])
       if "cuhnsw_amd::search_" in name:
         search += value
-        first_pass += ("search_fast_kernel" in name or "search_pair_kernel" in name)
+        first_pass += "search_fast_kernel" in name
       elif "copyBuffer" in name:
         copies.append(value)
     if not first_pass or not copies:
@@ -107,6 +107,116 @@ def workload_text(name, n, d, o, nq, k, ef, storage):
           if storage == "fp16" else "")
 
 
+def exact_topk(torch, data_dev, sq_dev, queries_dev, k, dot):
+  """Exact top-k on the GPU (harness only).  Scores are produced in blocks of at most 2^28 elements (1 GiB):
+  larger matmul outputs came back with wrong entries on this stack."""
+  n = data_dev.shape[0]
+  cols = 1 << 19
+  out = []
+  for s in range(0, queries_dev.shape[0], 512):
+    qs = queries_dev[s:s + 512]
+    best_v = best_i = None
+    for c in range(0, n, cols):
+      score = -(qs @ data_dev[c:c + cols].T)
+      if not dot:
+        score = sq_dev[None, c:c + cols] + 2.0 * score
+      tv, ti = torch.topk(score, min(k, score.shape[1]), dim=1, largest=False)
+      ti = ti + c
+      if best_v is not None:
+        tv, ti = torch.cat([best_v, tv], 1), torch.cat([best_i, ti], 1)
+        tv, sel = torch.topk(tv, min(k, tv.shape[1]), dim=1, largest=False)
+        ti = torch.gather(ti, 1, sel)
+      best_v, best_i = tv, ti
+    out.append(best_i.cpu().numpy())
+  return np.concatenate(out)
+
+
+def other_workload_rows(torch, capi, datasets, orc, tmpdir, name, efs, n_check=1000, n_recall=1000, steps=3):
+  """One of the other benchmark configurations at its full size, compactly: build seconds, and per ef_search the
+  search time of the whole batch (device pointers, HIP events on the engine's stream), QPS, recall, the
+  distance-gather roofline fraction counted like the headline's (distinct evaluations of a literal-only pass
+  x row bytes), the queries the literal pass answered, and the id rows that differ from the CPU oracle's on the
+  first n_check queries of the index file the GPU wrote (orc = None: no CPU check)."""
+  data, queries, spec = datasets.make(name)
+  o = spec["opt"]
+  n, d = data.shape
+  nq, k = queries.shape[0], spec["topk"]
+  dot = o["dist_type"] == "dot"
+  mult = o.get("level_mult") or 1.0 / np.log(o["max_m"])
+  levels = datasets.random_levels(n, mult)
+  opt = dict(seed=777, c_log_level=2, py_log_level=2, max_m=o["max_m"], max_m0=o["max_m0"],
+             ef_construction=o["ef_construction"], level_mult=mult, save_remains=False, hyper_threads=10.0,
+             block_dim=32, dist_type=o["dist_type"], visited_table_size=0, visited_list_size=8192, nrz=False,
+             reverse_cand=False, heuristic_coef=0.0)
+  opt_path = os.path.join(tmpdir, "opt_%s.json" % name)
+  with open(opt_path, "w") as f:
+    json.dump(opt, f)
+  eng = capi.Engine()
+  assert eng.init(opt_path) == 0
+  # the first launch of a kernel pays for loading its code: a small build and search of the same shape first
+  m = min(n, 20000)
+  eng.set_data(data[:m])
+  eng.set_random_levels(levels[:m])
+  eng.build_graph()
+  eng.search_knn(queries[:64], k, efs[-1])
+  eng.set_data(data)
+  eng.set_random_levels(levels)
+  eng.build_graph()
+  build_s = eng.last_build_seconds
+  dd = torch.from_numpy(data).cuda()
+  qq = torch.from_numpy(queries).cuda()
+  sq = None if dot else (dd * dd).sum(1)
+  gt = exact_topk(torch, dd, sq, qq[:n_recall], k, dot)
+  del dd, sq
+  torch.cuda.empty_cache()
+  ix = None
+  if orc is not None:
+    idx_path = os.path.join(tmpdir, "other_%s.idx" % name)
+    eng.save_index(idx_path)
+    ix = orc.OracleIndex(o["dist_type"]).load(idx_path)
+    os.remove(idx_path)
+  nns = torch.empty((nq, k), dtype=torch.int32, device="cuda")
+  dist = torch.empty((nq, k), dtype=torch.float32, device="cuda")
+  found = torch.empty(nq, dtype=torch.int32, device="cuda")
+  stats = torch.zeros((nq, 4), dtype=torch.int32, device="cuda")
+  torch.cuda.synchronize()
+
+  def step(ef, with_stats=False):
+    return eng.search_knn_device(qq.data_ptr(), nq, k, ef, nns.data_ptr(), dist.data_ptr(), found.data_ptr(),
+                                 stats.data_ptr() if with_stats else None)
+
+  rows = []
+  for ef in efs:
+    ef = max(ef, k)
+    eng.set_tunable("fast_path", 0)
+    step(ef, with_stats=True)              # literal queues only: the distinct evaluations
+    n_dist = int(stats[:, 0].sum().item())
+    eng.set_tunable("fast_path", 1)
+    step(ef)
+    ms = float(np.mean([step(ef) for _ in range(steps)]))
+    handed = int(eng.last_search_repeats)
+    ids = nns.cpu().numpy()
+    recall = float(np.mean([len(set(a) & set(b)) / k for a, b in zip(ids[:n_recall], gt)]))
+    gather = n_dist * 4 * d
+    row = {"ef_search": ef, "search_ms": ms, "value": nq / (ms * 1e-3), "unit": "queries/s",
+           "recall_at_%d" % k: recall, "frac": gather / (ms * 1e-3) / 8e12, "algorithmic_bytes_per_launch": gather,
+           "queries_repeated_with_literal_queues": handed}
+    if ix is not None:
+      n_c = min(nq, n_check)
+      o_ids, _, o_f = ix.search(queries[:n_c], k, ef, threads=orc.host_threads())
+      row["oracle_rows_checked"] = n_c
+      row["rows_with_id_mismatch_vs_oracle"] = int(((o_ids != ids[:n_c]).any(axis=1) |
+                                                    (o_f != found[:n_c].cpu().numpy())).sum())
+    rows.append(row)
+  out = {"workload": "%s: %dx%d %s max_m=%d max_m0=%d ef_construction=%d; %d queries topk=%d" % (
+             name, n, d, o["dist_type"], o["max_m"], o["max_m0"], o["ef_construction"], nq, k),
+         "build_seconds": build_s, "rows": rows}
+  eng.close()
+  del ix, qq, nns, dist, found, stats, data, queries
+  torch.cuda.empty_cache()
+  return out
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -124,14 +234,13 @@ def main():
                   help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
   ap.add_argument("--fast-path", type=int, default=1, choices=[0, 1, 2],
                   help="0 = literal priority queues only, 1 = default, 2 = sorted-set first pass whatever the batch size")
-  ap.add_argument("--pair-path", type=int, default=1, choices=[0, 1, 2],
-                  help="2 = two queries per wavefront in the first pass wherever the shapes allow it, 0 = never, 1 = the engine's choice (at present: never)")
   ap.add_argument("--query-order", type=int, default=1, choices=[0, 1, 2],
                   help="0 = queries in the caller's order, 1 = longest first from one to one and a half rounds of wavefronts on, 2 = from one")
   ap.add_argument("--trails", type=int, default=1, choices=[0, 1, 2],
                   help="0 = the literal pass searches handed-over queries from the entry point, 1 = from the first pass's "
                        "trail in batches of up to two rounds of wavefronts (default), 2 = in every batch")
   ap.add_argument("--no-large", action="store_true", help="skip the extra 4x batch (profiling runs)")
+  ap.add_argument("--no-others", action="store_true", help="skip the compact rows of the other benchmark configurations")
   ap.add_argument("--profile", action="store_true",
                   help="profiling run: only searches of the default path are launched (no literal-only counting pass, "
                        "no CPU baseline, no 4x batch); per_query and roofline then use the evaluations performed")
@@ -141,7 +250,7 @@ def main():
                   help="no benchmark: write profiles/hbm_traffic.json from two rocprofv3 --pmc output directories")
   args = ap.parse_args()
   if args.profile:
-    args.no_cpu = args.no_large = True
+    args.no_cpu = args.no_large = args.no_others = True
   if args.ingest_pmc:
     from cuhnsw_amd import datasets
     spec = datasets.CONFIGS[args.workload]
@@ -198,35 +307,16 @@ def main():
   eng.set_random_levels(levels)
   eng.build_graph()                      # the timed build (same graph: the build is deterministic)
   build_s = eng.last_build_seconds
-  eng.set_tunable("pair_path", args.pair_path)
   eng.set_tunable("query_order", args.query_order)
   eng.set_tunable("trails", args.trails)
 
-  # exact top-k on the GPU (harness only) for recall.  Scores are produced in blocks of at most
-  # 2^28 elements (1 GiB): larger matmul outputs came back with wrong entries on this stack.
+  # exact top-k on the GPU (harness only) for recall, measured on the first 20 000 queries of larger batches
   dd = torch.from_numpy(data).cuda()
   qq = torch.from_numpy(queries).cuda()
   sq = (dd * dd).sum(1) if o["dist_type"] != "dot" else None
-  cols = 1 << 19
-  gt = []
-  n_gt = min(nq, 20000)   # recall is measured on the first 20 000 queries of larger batches
-  for s in range(0, n_gt, 512):
-    qs = qq[s:min(s + 512, n_gt)]
-    best_v = best_i = None
-    for c in range(0, n, cols):
-      score = -(qs @ dd[c:c + cols].T)
-      if sq is not None:
-        score = sq[None, c:c + cols] + 2.0 * score
-      tv, ti = torch.topk(score, min(k, score.shape[1]), dim=1, largest=False)
-      ti = ti + c
-      if best_v is not None:
-        tv, ti = torch.cat([best_v, tv], 1), torch.cat([best_i, ti], 1)
-        tv, sel = torch.topk(tv, min(k, tv.shape[1]), dim=1, largest=False)
-        ti = torch.gather(ti, 1, sel)
-      best_v, best_i = tv, ti
-    gt.append(best_i.cpu().numpy())
-  gt = np.concatenate(gt)
-  del dd, score, sq
+  n_gt = min(nq, 20000)
+  gt = exact_topk(torch, dd, sq, qq[:n_gt], k, o["dist_type"] == "dot")
+  del dd, sq
 
   nns = torch.empty((nq, k), dtype=torch.int32, device="cuda")
   dist = torch.empty((nq, k), dtype=torch.float32, device="cuda")
@@ -321,7 +411,7 @@ def main():
   # two rocprofv3 --pmc runs of this script; null when that file was measured on another workload or on
   # other kernel sources (it cannot be measured from inside this process)
   wl = workload_text(args.workload, n, d, o, nq, k, ef, args.storage) + ("; rows padded to 16 bytes" if args.tight_rows else "")
-  traffic = measured_traffic(wl) if args.fast_path == 1 and args.pair_path == 1 else None
+  traffic = measured_traffic(wl) if args.fast_path == 1 else None
   achieved = gather_bytes / (avg_kernel_ms * 1e-3) / 1e9
   out = {
       "metric": "batch search QPS at recall@%d (%s: %dx%d %s), with build seconds" % (
@@ -344,8 +434,7 @@ def main():
                     "of_them_replayed_from_the_first_pass_trail": int(from_trails)},
       "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s",
                    "frac": achieved / 8000.0, "traffic": traffic,
-                   "kernel": ("search_pair_kernel" if (args.pair_path == 2 and d <= 128 and ef <= 128) else "search_fast_kernel") +
-                             " with search_kernel beside it (one search of the batch)"
+                   "kernel": "search_fast_kernel with search_kernel beside it (one search of the batch)"
                              if args.fast_path else "search_kernel (literal priority queues only)",
                    "algorithmic_bytes_per_launch": gather_bytes},
       "host_pointer_search": {"ms_per_call": host_ms, "value": nq / (host_ms * 1e-3), "unit": "queries/s",
@@ -418,6 +507,19 @@ def main():
                      "queries_meeting_equal_distances": int(tied.sum()),
                      "id_mismatches_among_them": int((bad_rows & tied).sum()),
                      "id_mismatches_among_the_rest": int((bad_rows & ~tied).sum())}
+  # the other benchmark configurations at full size, one compact block (the headline stays the workload above)
+  if args.workload == "C2" and args.n is None and args.nq is None and not args.no_others:
+    orc_mod = None
+    if not args.no_cpu:
+      from oracle import oracle as orc_mod
+    eng.close()
+    del eng, nns, dist, found, stats, qq, data, queries
+    torch.cuda.empty_cache()
+    t0 = time.time()
+    out["other_workloads"] = [
+        other_workload_rows(torch, capi, datasets, orc_mod, tmpdir, name, efs)
+        for name, efs in (("C1", [300]), ("C3", [64, 128, 300]), ("C4", [300]), ("C5", [128, 256, 512]))]
+    out["other_workloads_seconds"] = time.time() - t0
   print(json.dumps(out))
 
 
