@@ -18,6 +18,7 @@ SYMBOLS = [
     "cuhnsw_last_build_seconds", "cuhnsw_last_search_repeats", "cuhnsw_set_tunable",
     "cuhnsw_search_knn_device_noalloc", "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
     "cuhnsw_last_build_counters", "cuhnsw_debug_gather_probe", "cuhnsw_last_search_trails",
+    "cuhnsw_last_search_side_by_side", "cuhnsw_literal_fallbacks", "cuhnsw_trails_available",
 ]
 
 _lib = None
@@ -57,6 +58,9 @@ def load():
   l.cuhnsw_last_build_seconds.restype = cd
   l.cuhnsw_last_search_repeats.argtypes = [vp]
   l.cuhnsw_last_search_trails.argtypes = [vp]
+  l.cuhnsw_last_search_side_by_side.argtypes = [vp]
+  l.cuhnsw_literal_fallbacks.argtypes = [vp]
+  l.cuhnsw_trails_available.argtypes = [vp]
   l.cuhnsw_set_tunable.argtypes = [vp, ctypes.c_char_p, cd]
   _lib = l
   return l
@@ -177,4 +181,7 @@ class Engine:
   last_build_seconds = property(lambda s: s._l.cuhnsw_last_build_seconds(s._h))
   last_search_repeats = property(lambda s: s._l.cuhnsw_last_search_repeats(s._h))
   last_search_trails = property(lambda s: s._l.cuhnsw_last_search_trails(s._h))
+  last_search_side_by_side = property(lambda s: bool(s._l.cuhnsw_last_search_side_by_side(s._h)))
+  literal_fallbacks = property(lambda s: s._l.cuhnsw_literal_fallbacks(s._h))
+  trails_available = property(lambda s: bool(s._l.cuhnsw_trails_available(s._h)))
   last_build_dropped_links = property(lambda s: s._l.cuhnsw_last_build_dropped_links(s._h))

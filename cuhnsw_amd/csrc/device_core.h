@@ -1112,7 +1112,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
       accepted = 0ull;
     }
     if (gave_up) {
-      trail_stop(tr, st.n_hops - 1, st.n_dist);  // (a trail still recording here: the hop under way is not on it)
+      trail_stop(tr, st.n_hops - 1, st.n_dist - n);  // (a trail still recording here: the hop under way, and its evaluations, are not on it)
       break;
     }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
@@ -1282,11 +1282,16 @@ __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec
           if (mine) {
             s.nbuf[lane] = r.y;
             s.dbuf[lane] = __uint_as_float(r.z);
-            // (the filter learns the node: a later hop this pass makes itself need not evaluate it again)
-            uint2* sets = reinterpret_cast<uint2*>(s.vcache);
-            const int set_bits = s.vc_bits - 1;
-            const uint32_t slot = r.y & ((1u << set_bits) - 1u);
-            sets[slot] = filter_push(sets[slot], r.y >> set_bits);
+          }
+          // the filter learns the nodes (a later hop this pass makes itself need not evaluate them again), one
+          // lane after the other: two records of a hop may fall into the same set of tags
+          uint2* sets = reinterpret_cast<uint2*>(s.vcache);
+          const int set_bits = s.vc_bits - 1;
+          for (unsigned long long pend = run; pend != 0ull; pend &= pend - 1ull) {
+            if (lane == __builtin_ctzll(pend)) {
+              const uint32_t slot = r.y & ((1u << set_bits) - 1u);
+              sets[slot] = filter_push(sets[slot], r.y >> set_bits);
+            }
           }
           trail_at += n;
           from_trail = true;

@@ -10,9 +10,11 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -62,11 +64,15 @@ static __device__ __align__(256) unsigned char scratch[sizeof(StaticScratch)];  
 
 constexpr int kMaxDevices = 64;
 static StaticScratch* g_static_scratch[kMaxDevices] = {};
+static std::mutex g_static_scratch_mutex;             // guards the table above
+static std::atomic_flag g_static_busy[kMaxDevices];   // set while a no-allocation search uses the device's array
 // device address of this device's copy of `scratch`; looked up on first use, then kept
-static StaticScratch* static_scratch_for_current_device() {
+static StaticScratch* static_scratch_for_current_device(int* device = nullptr) {
   int dev = 0;
   HIP_CHECK(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) throw std::runtime_error("device ordinal beyond the table of static scratch addresses");
+  if (device) *device = dev;
+  std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
   if (!g_static_scratch[dev]) {
     void* ptr = nullptr;
     HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
@@ -74,8 +80,20 @@ static StaticScratch* static_scratch_for_current_device() {
   }
   return g_static_scratch[dev];
 }
+// One no-allocation search at a time per GPU: every engine of the process shares that GPU's array.
+struct StaticScratchLease {
+  int dev;
+  explicit StaticScratchLease(int d) : dev(d) {
+    if (g_static_busy[dev].test_and_set(std::memory_order_acquire))
+      throw std::runtime_error("search_knn (no allocation): another no-allocation search is running on this GPU "
+                               "(all engines of a process share the GPU's scratch array; serialise the calls)");
+  }
+  ~StaticScratchLease() { g_static_busy[dev].clear(std::memory_order_release); }
+  StaticScratchLease(const StaticScratchLease&) = delete;
+  StaticScratchLease& operator=(const StaticScratchLease&) = delete;
+};
 
-// (a fill kernel rather than hipMemsetAsync: a caller may record the no-allocation search into a HIP graph)
+// (the no-allocation search clears its control words with this kernel: it issues no memset)
 __global__ void __launch_bounds__(128) fill_ints_kernel(int* p, int n, int value) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = value;
@@ -96,6 +114,18 @@ struct DevBuf {
     release();
     HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&p), want * sizeof(T)));
     n = want;
+  }
+  // the same for a buffer the caller can do without: false (and an empty buffer) when the memory is not there
+  bool try_reserve(size_t want) {
+    if (want <= n) return true;
+    release();
+    if (hipMalloc(reinterpret_cast<void**>(&p), want * sizeof(T)) != hipSuccess) {
+      (void)hipGetLastError();
+      p = nullptr;
+      return false;
+    }
+    n = want;
+    return true;
   }
   ~DevBuf() { release(); }
 };
@@ -127,9 +157,16 @@ class Engine {
   bool share_known = false;               // last_repeat_share comes from a search of this index
   double last_repeat_share = 0.0;         // its wavefronts per CU
   int concurrent_literal = 1;  // run the literal pass beside the sorted-set pass (0: after it)
+  // A literal wavefront whose bounded wait ran out (the two streams did not run side by side: a profiler that
+  // serialises kernels, a saturated device) makes the next kSequentialSearches searches run their passes one
+  // after the other; then the concurrent schedule is tried again.  The caller's setting above is left alone.
+  static constexpr int kSequentialSearches = 8;
+  int sequential_left = 0;       // searches still to run one pass after the other
+  int literal_fallbacks = 0;     // how often that happened on this index
+  int last_side_by_side = 0;     // the last search ran its literal pass beside the first pass
+  bool trails_unavailable = false;  // the trail buffers could not be allocated: searches go on without trails
   int filter_entries = 0;  // entries of the sorted-set search's visited filter (0 = automatic)
   int first_pass_waves = 0;  // wavefronts per CU of the first pass (0 = as many as fit)
-  int pair_path = 1;       // first pass with two queries per wavefront: 2 = where the shapes allow it, 0 / 1 = never (1: automatic)
   int query_order = 1;     // first pass of 1.5 to 32 rounds of wavefronts: longest queries first (0: caller's order)
   bool fast_suspended = false;  // this index ties too often for the sorted-set search to pay (integer data)
   int lean_literal = 1;  // literal pass: 0 = always the exact visited bitmap, 1 = automatic, 2 = always the LDS filter
@@ -175,6 +212,7 @@ class Engine {
   DevBuf<float> d_q, d_dist;
   DevBuf<int> d_nns, d_found;
   StaticScratch* static_scratch = nullptr;  // this device's copy (device address)
+  int device_ordinal = 0;
   int* h_ctl = nullptr;                     // pinned: control words read back without staging
   long long wall_clock_khz = 100000;        // ticks of wall_clock64() per millisecond
 
@@ -189,7 +227,7 @@ class Engine {
       int khz = 0;
       if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) == hipSuccess && khz > 0) wall_clock_khz = khz;
       else (void)hipGetLastError();
-      static_scratch = static_scratch_for_current_device();
+      static_scratch = static_scratch_for_current_device(&device_ordinal);
       HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_ctl), 64 * sizeof(int), hipHostMallocDefault));
       HIP_CHECK(hipStreamCreate(&stream));
       HIP_CHECK(hipEventCreate(&ev0));
@@ -292,6 +330,7 @@ class Engine {
     host.D = d;
     host.vectors.assign(data, data + (size_t)n * d);
     have_levels = have_graph = host_links_stale = false;
+    forget_search_history();
     pool_slots = 0;  // the slot pool is sized by N: rebuild it lazily
     pool = SlotPool{};
     if (has_device) upload_vectors();  // without a GPU only the host-side calls remain usable
@@ -336,6 +375,33 @@ class Engine {
     have_levels = true;
     have_graph = false;
     if (has_device) upload_structure();
+  }
+
+  // What a search learns about an index (how many of its queries tie, whether the two passes ran side by
+  // side) belongs to that index: forgotten whenever another one takes its place.
+  void forget_search_history() {
+    fast_suspended = false;
+    share_known = false;
+    last_repeat_share = 0.0;
+    sequential_left = 0;
+    literal_fallbacks = 0;
+    last_side_by_side = 0;
+    last_repeats = last_trails = 0;
+  }
+
+  // Buffers of a search that do not depend on the batch are allocated when the index becomes resident, not
+  // inside the first search that wants them: the trails of the sorted-set pass (one buffer per wavefront the
+  // GPU can hold plus the spares).  They are an optimisation: if the memory is not there the searches go on
+  // without trails.
+  size_t trail_records_wanted(int slots) const { return (size_t)(slots + trail_spares) * (size_t)trail_cap; }
+  void reserve_trails(int slots) {
+    if (!trails || trails_unavailable) return;
+    if (!d_trail.try_reserve(trail_records_wanted(slots))) trails_unavailable = true;
+  }
+  void prepare_search_buffers() {
+    if (!has_device) return;
+    trails_unavailable = false;
+    reserve_trails(28 * num_cus);  // seven wavefronts per SIMD: what the sorted-set pass holds at most where it keeps trails
   }
 
   // ---- slots -----------------------------------------------------------------------------
@@ -495,24 +561,8 @@ class Engine {
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
       auto fast_kernel = search_fast_kernel<DT, QR, NS>;
-      // two queries per wavefront where the query fits two float4 registers per lane, a link row fits a
-      // half's 32 lanes and the sorted set fits 32 lanes' registers
-      constexpr bool kPairShape = (QR == 1 || QR == 2) && NS == 2;
-      constexpr int N2 = kPairShape ? 2 * NS : 2;
-      auto pair_kernel = search_pair_kernel<DT, (kPairShape ? QR : 1), N2>;
-      // (pair_path = 2 asks for it.  It used to be the faster kernel at ef_search up to 64, and up to 128 on batches
-      // of several rounds of wavefronts — 1.18 M x 50, 40 000 queries, ef 128: 5.5 against 6.5 ms.  Against the
-      // one-query kernel as it is built now it no longer is, anywhere measured: 1.18 M x 50, 40 000 queries, ef 32 /
-      // 64 / 128: 2.68 / 3.20 / 4.40 ms against 2.70 / 3.08 / 3.99; 10 M x 96, 100 000 queries, ef 64 / 128: 16.4 /
-      // 18.5 against 14.1 / 15.4 ms; 1 M x 128, 10 000 queries, ef 64: 2.10 against 1.62 ms.  So the automatic
-      // setting, pair_path = 1, does not choose it at present.)
-      const bool pair = kPairShape && pair_path > 1 && !a.reverse && host.S0 <= 32 && host.SU <= 32 && a.nq > 1;
-      auto fast_lds = [&](int bits) -> size_t {
-        return pair ? plan_pair_lds(a.lcap, bits).total : plan_fast_lds(QR, ix.Dp, a.lcap, bits).total;
-      };
-      auto fast_slots = [&](int bits) -> int {
-        return pair ? resident_slots(pair_kernel, fast_lds(bits)) : resident_slots(fast_kernel, fast_lds(bits));
-      };
+      auto fast_lds = [&](int bits) -> size_t { return plan_fast_lds(QR, ix.Dp, a.lcap, bits).total; };
+      auto fast_slots = [&](int bits) -> int { return resident_slots(fast_kernel, fast_lds(bits)); };
       // the filter must not be what limits the wavefronts per CU: half the filter repeats more
       // evaluations but is the faster choice wherever it buys occupancy (10 M x 96, ef = 512,
       // five wavefronts per SIMD by registers: 46.8 ms with 8 KB of filter, 45.2 ms with 4 KB)
@@ -524,7 +574,8 @@ class Engine {
       }
       const size_t fast_lds_bytes = fast_lds(a.fc_bits);
       int slots = fast_slots(a.fc_bits);
-      const bool side = concurrent_literal && max_slots_override <= 0;
+      const bool side = concurrent_literal && sequential_left == 0 && max_slots_override <= 0;
+      last_side_by_side = side ? 1 : 0;
       int side_slots = 0;
       // few queries need the literal pass (0.4 % of the 1.18M-point set's): one wavefront per CU
       // serves them without taking room from the first pass; two when the last search needed more
@@ -541,7 +592,7 @@ class Engine {
       }
       if (max_slots_override > 0) slots = max_slots_override;
       if (first_pass_waves > 0) slots = std::min(slots, first_pass_waves * num_cus);
-      slots = std::max(1, std::min(slots, pair ? (a.nq + 1) / 2 : a.nq));
+      slots = std::max(1, std::min(slots, a.nq));
       HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 128 * sizeof(int), stream));
       HIP_CHECK(hipMemsetAsync(d_redo.p, 0xFF, (size_t)a.nq * sizeof(int), stream));
       // (every allocation before the literal pass is launched: growing a buffer frees the old one, and
@@ -550,7 +601,7 @@ class Engine {
       // 12 000 queries, 1.7 rounds: 3.10 -> 2.85 ms on average; of 10 000, 1.4 rounds: 2.92 and 2.96 — the first
       // pass alone gains, 2.8 -> 2.2 ms, but the one query in ten thousand that is handed over then tends to be
       // one that ends last; query_order = 2 puts any batch of more than one round in order)
-      const long long resident = pair ? 2LL * slots : slots;  // queries at work at a time
+      const long long resident = slots;  // queries at work at a time
       // (and up to 32 rounds: what the order saves is part of one round, what the separate descents cost grows
       // with the batch — 1 000 000 queries, 145 rounds: 211.7 against 201.9 ms in the caller's order)
       // A handed-over query is not searched again from its entry point: the first pass leaves the entries it
@@ -560,8 +611,16 @@ class Engine {
       // trail costs the first pass 2 to 3 %, which only a batch short enough to wait for its last hand-over
       // gets back (1.18 M x 50, longest first, eight draws of 10 000 queries: 2.75 -> 2.65 ms on average, the
       // slowest draws 3.06 -> 2.88; 40 000 queries: 6.24 -> 6.39 ms with trails kept).  trails = 2: whatever the batch.
-      const bool keep_trails = (QR == 1 || QR == 2) && trails && !pair && !a.reverse && a.lean && host.S0 <= 63 &&
-                               (trails > 1 || a.nq <= 2 * resident);
+      bool keep_trails = (QR == 1 || QR == 2) && trails && !a.reverse && a.lean && host.S0 <= 63 &&
+                         (trails > 1 || a.nq <= 2 * resident);
+      if (keep_trails) {
+        // (normally there since the index became resident; a changed trail_cap / trail_spares asks again)
+        if (d_trail.n < trail_records_wanted(slots)) {
+          trails_unavailable = false;
+          reserve_trails(slots);
+        }
+        keep_trails = !trails_unavailable && d_trail.n >= trail_records_wanted(slots);
+      }
       // (with trails a late hand-over costs less, and the order pays from one round on)
       const bool in_order = query_order && (query_order > 1 ? a.nq > resident
                                                              : (keep_trails ? a.nq > resident : 2 * a.nq >= 3 * resident) &&
@@ -572,7 +631,6 @@ class Engine {
         d_order_hist.reserve((size_t)kOrderBuckets);
       }
       if (keep_trails) {
-        d_trail.reserve((size_t)(slots + trail_spares) * trail_cap);
         d_redo_trail.reserve((size_t)a.nq);
         a.trail = d_trail.p;
         a.trail_cap = trail_cap;
@@ -625,8 +683,7 @@ class Engine {
                            a.nq, d_order_hist.p, d_order.p);
         HIP_CHECK(hipGetLastError());
       }
-      if (pair) hipLaunchKernelGGL(pair_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
-      else hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
+      hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
       HIP_CHECK(hipGetLastError());
       if (side) {
         HIP_CHECK(hipStreamWaitEvent(stream, ev_side1, 0));
@@ -638,6 +695,7 @@ class Engine {
       last_trails = ctl[48];
       last_repeat_share = (double)n_literal / a.nq;
       share_known = true;
+      if (!side && sequential_left > 0) --sequential_left;
       // an index whose distances tie all the time (integer-valued data) sends most queries
       // through both passes: stop trying the sorted set on it
       if (a.nq >= 256 && (long long)n_literal * 3 > a.nq) fast_suspended = true;
@@ -646,9 +704,12 @@ class Engine {
         if (!answered) {
           scrub_pool();
           if (ctl[1] & 1) glob_cap *= 4;
-          // the wait ran out on its own bound: the streams of this process do not run side by side
-          // (a profiler collecting counters, a saturated device); from now on one pass after the other
-          if ((ctl[1] & 2) && spin_limit_override < 0) concurrent_literal = 0;
+          // the wait ran out: the streams of this process do not run side by side at present (a profiler
+          // collecting counters, a saturated device); the next searches run one pass after the other
+          if (ctl[1] & 2) {
+            sequential_left = kSequentialSearches;
+            ++literal_fallbacks;
+          }
         }
       }
     }
@@ -688,6 +749,7 @@ class Engine {
   template <int DT, int QR, int NS>
   void launch_search_static(const DevIndex& ix, SearchArgs& a, float* ms) {
     if constexpr (NS > 0) {
+      StaticScratchLease lease(device_ordinal);  // released on every way out of this function
       StaticScratch* sc = static_scratch;
       a.counter = sc->ctl;
       a.status = sc->ctl + 1;
@@ -750,11 +812,6 @@ class Engine {
   }
   template <int DT>
   void launch_search_qr(int q, int ns, const DevIndex& ix, SearchArgs& a, float* ms) {
-#ifdef CUHNSW_QUICK_BUILD  // experiments only: one query layout
-    if (q != 1) throw std::runtime_error("quick build: only queries of up to 64 dimensions");
-    launch_search_ns<DT, 1>(ns, ix, a, ms);
-    return;
-#endif
     switch (q) {
       case 1: launch_search_ns<DT, 1>(ns, ix, a, ms); break;
       case 2: launch_search_ns<DT, 2>(ns, ix, a, ms); break;
@@ -998,11 +1055,6 @@ class Engine {
   }
   template <int DT>
   void build_qr(int q, int ns) {
-#ifdef CUHNSW_QUICK_BUILD
-    if (q != 1) throw std::runtime_error("quick build: only vectors of up to 64 dimensions");
-    build_ns<DT, 1>(ns);
-    return;
-#endif
     switch (q) {
       case 1: build_ns<DT, 1>(ns); break;
       case 2: build_ns<DT, 2>(ns); break;
@@ -1023,8 +1075,8 @@ class Engine {
     else build_qr<DIST_L2>(q, ns);
     last_build_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     have_graph = true;
-    fast_suspended = false;
-    share_known = false;
+    forget_search_history();
+    prepare_search_buffers();
     host_links_stale = true;
   }
 
@@ -1068,8 +1120,7 @@ class Engine {
     if (fresh.N <= 0) throw std::runtime_error("load_index: empty index");
     host = std::move(fresh);
     have_data = have_levels = have_graph = true;
-    fast_suspended = false;
-    share_known = false;
+    forget_search_history();
     host_links_stale = false;
     if (has_device) {
       upload_vectors();
@@ -1080,6 +1131,7 @@ class Engine {
       HIP_CHECK(hipStreamSynchronize(stream));
       pool_slots = 0;  // N may have changed: rebuild the slot pool lazily
       pool = SlotPool{};
+      prepare_search_buffers();
     }
   }
 };
@@ -1091,6 +1143,7 @@ using cuhnsw_amd::Engine;
 
 struct cuhnsw_engine {
   Engine impl;
+  std::mutex mutex;  // calls on one engine are serialised: they share its staging buffers, slot pool and streams
 };
 
 namespace {
@@ -1099,6 +1152,7 @@ thread_local std::string g_create_error;
 template <typename F>
 int guarded(cuhnsw_engine* e, F&& f) {
   if (!e) return -1;
+  std::lock_guard<std::mutex> lock(e->mutex);
   try {
     e->impl.err.clear();
     f(e->impl);
@@ -1131,6 +1185,7 @@ const char* cuhnsw_last_error(cuhnsw_engine* e) { return e ? e->impl.err.c_str()
 
 int cuhnsw_init(cuhnsw_engine* e, const char* opt_path) {
   if (!e) return -1;
+  std::lock_guard<std::mutex> lock(e->mutex);
   return e->impl.init(opt_path);
 }
 int cuhnsw_set_data(cuhnsw_engine* e, const float* data, int num_data, int num_dims) {
@@ -1190,8 +1245,12 @@ int cuhnsw_has_device(void) { return cuhnsw_amd::device_present() ? 1 : 0; }
 double cuhnsw_last_build_seconds(cuhnsw_engine* e) { return e ? e->impl.last_build_seconds : 0.0; }
 int cuhnsw_last_search_repeats(cuhnsw_engine* e) { return e ? e->impl.last_repeats : 0; }
 int cuhnsw_last_search_trails(cuhnsw_engine* e) { return e ? e->impl.last_trails : 0; }
+int cuhnsw_last_search_side_by_side(cuhnsw_engine* e) { return e ? e->impl.last_side_by_side : 0; }
+int cuhnsw_literal_fallbacks(cuhnsw_engine* e) { return e ? e->impl.literal_fallbacks : 0; }
+int cuhnsw_trails_available(cuhnsw_engine* e) { return e ? (e->impl.trails_unavailable ? 0 : 1) : 0; }
 int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   if (!e || !name) return -1;
+  std::lock_guard<std::mutex> lock(e->mutex);
   std::string n(name);
   if (n == "build_batch") e->impl.build_batch = (int)value;
   else if (n == "level_first") e->impl.level_first = (int)value;
@@ -1206,7 +1265,6 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "trail_cap") e->impl.trail_cap = std::max(1, (int)value);
   else if (n == "trail_spares") e->impl.trail_spares = std::max(0, (int)value);
   else if (n == "filter_entries") e->impl.filter_entries = (int)value;
-  else if (n == "pair_path") e->impl.pair_path = (int)value;
   else if (n == "query_order") e->impl.query_order = (int)value;
   else if (n == "first_pass_waves") e->impl.first_pass_waves = (int)value;
   else if (n == "concurrent_literal") e->impl.concurrent_literal = value != 0.0;

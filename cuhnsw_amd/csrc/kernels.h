@@ -24,7 +24,6 @@
 //                      The result is deterministic for a given batch schedule.
 #pragma once
 #include "device_core.h"
-#include "pair_search.h"
 
 namespace cuhnsw_amd {
 
@@ -452,11 +451,14 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     if (gave_up) {
       // (the trail's records are written by many lanes: all of them out before lane 0 publishes the entry)
       const bool with_trail = a.redo_trail && trail_buf >= 0 && tr.n > 0 && tr.hops > 0;
+      // a search that went all the way (only the cut at k is open) and whose trail covers every hop: the literal
+      // pass needs no search at all, only the result heap replayed from the trail (hops stored negative)
+      const bool whole = how != 1 && tr.hops == st.n_hops;
       if (with_trail) __threadfence();
       int spare = 0;
       if (lane == 0) {
         const int slot = atomicAdd(a.repeats, 1);
-        if (a.redo_trail) a.redo_trail[slot] = make_int4(with_trail ? trail_buf : -1, tr.n, tr.hops, tr.n_dist);
+        if (a.redo_trail) a.redo_trail[slot] = make_int4(with_trail ? trail_buf : -1, tr.n, whole ? -tr.hops : tr.hops, tr.n_dist);
         __hip_atomic_store(&a.redo[slot], qi, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         if (with_trail) spare = atomicAdd(a.trail_next, 1);
       }
@@ -500,351 +502,6 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     __threadfence();
     if (lane == 0) atomicAdd(a.done, 1);
     wave_sync();
-  }
-}
-
-// First pass of a search batch with TWO queries per wavefront (pair_search.h): same answers, same give-up
-// list and counters as search_fast_kernel, which it replaces where the query fits two float4 registers per
-// lane, link rows fit 32 slots and ef fits 32*N entries.  N = sorted-set slots per lane.
-template <int DT, int QR, int N>
-__global__ void __launch_bounds__(64, N <= 4 ? 5 : 4) search_pair_kernel(DevIndex ix, SearchArgs a) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int lane = threadIdx.x;
-  const int hl = lane & 31;
-  const PairLdsPlan lp = plan_pair_lds(a.lcap, a.fc_bits);
-  unsigned char* mine = smem + (lane < 32 ? 0 : lp.half_bytes);
-  uint2* sets = reinterpret_cast<uint2*>(mine + lp.fcache);
-  uint32_t* nbuf = reinterpret_cast<uint32_t*>(mine + lp.nbuf);
-  float* dbuf = reinterpret_cast<float*>(mine + lp.dbuf);
-  const int set_bits = a.fc_bits - 1;
-  const uint32_t set_mask = (1u << set_bits) - 1u;
-  const int ef = a.ef;
-  if (blockIdx.x == 0 && lane == 0) __hip_atomic_store(a.done + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if (hl == 0) nbuf[0] = 0u;  // the distance pass reads ids[0] of a half that has nothing to evaluate
-  wave_sync();
-
-  // per-half state (the same value in the 32 lanes of a half)
-  int phase = PP_NEED, level = 0, qi = -1;
-  uint32_t cur = 0;
-  float dcur = 0.f;
-  int n_acc = 0;
-  float lower = 0.f, maxkey = -INFINITY;
-  bool have_tie = false, in_group = false, gave_up = false;
-  float group_key = 0.f, group_edge = INFINITY, ek_min = INFINITY;
-  // the twins of a single eviction out of two equal largest keys (see search_level_fast)
-  int ghosts = 0;
-  uint32_t ghost = kEmpty;
-  bool twin_phase = false;
-  const bool whole_set = a.k >= ef;
-  int n_dist = 0, n_hops = 0, n_dist_upper = 0, n_sweeps = 0;
-  QVec<QR> qv;
-#pragma unroll
-  for (int k = 0; k < QR; ++k) qv.q[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-  Frontier<N> fr;
-  pf_init<N>(fr, ef, hl);
-
-  for (;;) {
-    // ---- a half without a query takes the next one ------------------------------------------------------
-    if (wave_any(phase == PP_NEED)) {
-      int got = 0;
-      if (phase == PP_NEED && hl == 0) {
-        got = atomicAdd(a.counter, 1);
-        if (got < a.nq && a.order) got = a.order[got];  // longest queries first
-      }
-      got = half_read(got, 0, lane);
-      if (phase == PP_NEED) {
-        if (got >= a.nq) {
-          phase = PP_IDLE;
-        } else {
-          qi = got;
-          const float* src = a.q + (size_t)qi * ix.D;
-          const int sub = lane & 15;
-#pragma unroll
-          for (int k = 0; k < QR; ++k) {
-            const int i = 4 * (sub + 16 * k);
-            float4 t;
-            t.x = i + 0 < ix.D ? src[i + 0] : 0.0f;
-            t.y = i + 1 < ix.D ? src[i + 1] : 0.0f;
-            t.z = i + 2 < ix.D ? src[i + 2] : 0.0f;
-            t.w = i + 3 < ix.D ? src[i + 3] : 0.0f;
-            qv.q[k] = t;
-          }
-          n_acc = 0; lower = 0.f; maxkey = -INFINITY;
-          have_tie = false; in_group = false; gave_up = false;
-          group_key = 0.f; group_edge = INFINITY; ek_min = INFINITY;
-          ghosts = 0; ghost = kEmpty; twin_phase = false;
-          n_dist = 0; n_hops = 0; n_dist_upper = 0; n_sweeps = 0;
-          cur = ix.enterpoint;
-          phase = PP_ENTRY;
-          if (a.entry) {
-            // the descent through the upper levels has been done for the whole batch: straight to level 0,
-            // with a fresh sorted set and visited filter
-            const uint4 en = a.entry[qi];
-            cur = en.x;
-            n_dist_upper = (int)en.z;
-            n_sweeps = (int)en.w;
-            phase = PP_SEED;
-            pf_init<N>(fr, ef, hl);
-            uint4* c4 = reinterpret_cast<uint4*>(sets);
-            const int n4 = (1 << a.fc_bits) >> 2;
-            for (int i = hl; i < n4; i += 32) c4[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
-          }
-        }
-      }
-    }
-    if (!wave_any(phase != PP_IDLE)) break;
-
-    // ---- the step's id list ----------------------------------------------------------------------------------
-    bool ending = false;
-    int cid = -1;
-    if (wave_any(phase == PP_SEARCH)) {
-      cid = pf_take<N>(fr, phase == PP_SEARCH, lane);
-      if (wave_any(phase == PP_SEARCH && have_tie)) {
-        const bool on = phase == PP_SEARCH && have_tie;
-        const float d = cid >= 0 ? pf_key_of<N>(fr, (uint32_t)(cid >= 0 ? cid : 0), lane) : INFINITY;
-        const bool open = pf_open_key<N>(fr, d, lane);
-        if (on && in_group && cid >= 0 && d < group_key) {
-          // a closer candidate inside the group: expanded before the rest of it under any order; a group
-          // within the group is not followed
-          gave_up = open;
-        } else if (on && in_group && d != group_key) {
-          // the group is through: with another order of its members an offer or an entry whose key equals
-          // the bound reached now could have ended up on the other side of it, and with the bound below the
-          // group's key a member popped late would not have been expanded at all
-          gave_up = n_acc >= ef && (group_edge == lower || lower < group_key);
-          in_group = false;
-        }
-        if (on) {
-          if (cid >= 0) {
-            if (d >= ek_min) {
-              // the twin the set kept: the set's last entry, its key is the bound
-              if (ghosts == 1 && !in_group && !open) twin_phase = true;
-              else gave_up = true;
-            }
-            if (!in_group && !twin_phase) {
-              in_group = open;  // other waiting entries with this very key
-              group_key = d;
-              group_edge = INFINITY;
-            }
-          } else if (!gave_up && n_acc >= ef && lower >= ek_min) {
-            if (ghosts == 1) {
-              if ((ghost & kExpanded) == 0u) {
-                cid = (int)ghost;  // the twin the set pushed out: expanded, nothing of it may be accepted
-                ghost |= kExpanded;
-                twin_phase = true;
-              }
-            } else {
-              gave_up = true;
-            }
-          }
-        }
-      }
-      ending = phase == PP_SEARCH && (gave_up || cid < 0);
-      if (phase == PP_SEARCH && !ending) n_hops += 1;
-    }
-    const bool row_step = (phase == PP_SEARCH && !ending) || phase == PP_DESCEND;
-    int n = 0;
-    {
-      wave_sync();
-      // link row of the step (any valid row for a half that reads none)
-      const bool lvl0 = phase != PP_DESCEND;
-      const uint32_t node = row_step ? (phase == PP_SEARCH ? (uint32_t)cid : cur) : 0u;
-      const int S = lvl0 ? ix.S0 : ix.SU;
-      const uint32_t* row = lvl0 ? ix.links0 + (size_t)node * ix.S0
-                                 : ix.linksU + (size_t)(ix.upper_off[row_step ? node : ix.enterpoint] + level - 1) * ix.SU;
-      uint32_t id = kEmpty;
-      if (row_step) {
-        const uint32_t got = row[hl < S ? hl : 0];
-        id = hl < S ? got : kEmpty;
-      }
-      if (phase == PP_ENTRY || phase == PP_SEED) id = hl == 0 ? cur : kEmpty;
-      bool ask = id != kEmpty;
-      if (ask && (phase == PP_SEARCH || phase == PP_SEED)) {
-        const uint32_t slot = id & set_mask;
-        const uint32_t tag = id >> set_bits;
-        const uint2 w = sets[slot];
-        ask = (w.x & 0xFFFFu) != tag && (w.x >> 16) != tag && (w.y & 0xFFFFu) != tag && (w.y >> 16) != tag;
-        if (ask) sets[slot] = filter_push(w, tag);
-      }
-      const uint32_t m = half_ballot(ask, lane);
-      if (ask) nbuf[__popc(m & ((1u << hl) - 1u))] = id;
-      n = __popc(m);
-      if (phase == PP_DESCEND) n_sweeps += 1;
-      wave_sync();
-    }
-
-    // ---- keys ------------------------------------------------------------------------------------------------------
-    pair_dist<DT, QR, false>(ix, qv, nbuf, n, dbuf, lane);
-    if (phase == PP_DESCEND || phase == PP_ENTRY) n_dist_upper += phase == PP_DESCEND ? n : 0;
-    else n_dist += n;
-    wave_sync();
-
-    // ---- consumers ------------------------------------------------------------------------------------------------
-    const float my_key = hl < n ? dbuf[hl < n ? hl : 0] : INFINITY;
-    if (phase == PP_ENTRY) {
-      dcur = half_read(my_key, 0, lane);
-    }
-    if (wave_any(phase == PP_DESCEND)) {
-      // the strictly closest entry of the list captured at the sweep's start: first occurrence of the minimum
-      const float best = half_min(my_key);
-      const uint32_t at = half_ballot(my_key == best, lane);
-      const uint32_t to = nbuf[__builtin_ctz(at | 0x80000000u) & 31];
-      if (phase == PP_DESCEND) {
-        if (n > 0 && best < dcur) {
-          dcur = best;
-          cur = to;  // and sweep again on this level
-        } else {
-          level -= 1;
-        }
-      }
-    }
-    if (wave_any(phase == PP_SEARCH || phase == PP_SEED)) {
-      const bool searching = phase == PP_SEARCH || phase == PP_SEED;
-      const bool pass = searching && hl < n && (n_acc < ef || lower > my_key);
-      uint32_t todo = half_ballot(pass, lane);
-      if (wave_any(searching && in_group))
-        group_edge = (searching && in_group) ? fminf(group_edge, half_min((hl < n && !pass) ? my_key : INFINITY)) : group_edge;
-      while (wave_any(todo != 0u)) {
-        const bool valid = todo != 0u;
-        const int j = __builtin_ctz(todo | 0x80000000u) & 31;
-        todo &= todo - 1u;
-        const float key = dbuf[j];
-        const uint32_t id = nbuf[j];
-        const bool acc = valid && (n_acc < ef || lower > key);
-        // an eviction out of several equal largest keys: the heap's choice decides which of them stays in
-        // the result set, and the other one stays a live candidate of hnswlib
-        bool twins = false;
-        uint32_t last = kEmpty;  // the entry a full set is about to push out
-        if (wave_any(acc && have_tie && n_acc >= ef)) {
-          twins = acc && have_tie && n_acc >= ef && pf_max_twice<N>(fr, lane);
-          last = (uint32_t)__builtin_bit_cast(int, half_last(__builtin_bit_cast(float, (int)fr.v[N - 1]), lane));
-        }
-        const int r = pf_insert<N>(fr, key, id, acc, lane);
-        const bool ins = acc && r != 2;
-        if (wave_any(ins && twins)) {
-          const bool still = pf_max_twice<N>(fr, lane);
-          if (ins && twins) {
-            ek_min = fminf(ek_min, lower);
-            ghost = last;
-            ghosts += (still || whole_set) ? 2 : 1;  // three equal largest keys, a second event, the whole set asked for
-          }
-        }
-        if (ins && twin_phase) {
-          gave_up = true;  // which twin hnswlib expands first now decides whether the other one is expanded at all
-          todo = 0u;
-        }
-        have_tie = have_tie || (ins && r == 1);
-        if (ins && in_group && n_acc >= ef) {
-          group_edge = fminf(group_edge, lower);  // the entry this insert evicted
-          // a member of the group pushed out before its turn: with another order it would have been expanded
-          if (lower == group_key && (last & kExpanded) == 0u) {
-            gave_up = true;
-            todo = 0u;
-          }
-        }
-        if (valid && !acc && in_group) group_edge = fminf(group_edge, key);
-        n_acc += ins ? 1 : 0;
-        maxkey = ins ? fmaxf(maxkey, key) : maxkey;
-        const float top = pf_max<N>(fr, lane);
-        lower = ins ? (n_acc >= ef ? top : maxkey) : lower;  // hnswlib's lowerBound
-      }
-      ending = ending || (searching && gave_up);
-    }
-
-    // ---- phase changes ------------------------------------------------------------------------------------------
-    if (phase == PP_SEED) phase = PP_SEARCH;
-    if (phase == PP_ENTRY) {
-      level = ix.maxlevel;
-      phase = PP_DESCEND;
-    }
-    if (phase == PP_DESCEND && level <= 0) {
-      phase = PP_SEED;
-      // a fresh sorted set and visited filter for the level-0 search
-      pf_init<N>(fr, ef, hl);
-      uint4* c4 = reinterpret_cast<uint4*>(sets);
-      const int n4 = (1 << a.fc_bits) >> 2;
-      for (int i = hl; i < n4; i += 32) c4[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
-    }
-
-    // ---- a query ends: answer it, or hand it to the literal pass ------------------------------------------
-    if (wave_any(ending)) {
-      wave_sync();
-      const int top_size = n_acc < ef ? n_acc : ef;
-      const int T = top_size < a.k ? top_size : a.k;
-      const bool tied = ending && !gave_up && have_tie;
-      // Equal keys across the cut at k: which of them stays is up to the result heap, which the literal
-      // search reproduces.  Equal keys among the k best: the answer lists them by label.
-      const bool cut_tie = pf_tie_within<N>(fr, ef, T, top_size, T - 1, lane) && tied;
-      const bool inner_tie = pf_tie_within<N>(fr, ef, T - 1, top_size, 0, lane) && tied;
-      const bool hand_over = ending && (gave_up || cut_tie || (inner_tie && T > (1 << a.fc_bits)));
-      const bool answer = ending && !hand_over;
-      if (hand_over && hl == 0) {
-        const int slot = atomicAdd(a.repeats, 1);
-        __hip_atomic_store(&a.redo[slot], qi, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      pf_dump<N>(fr, ef, T, nbuf, dbuf, answer, lane);
-      wave_sync();
-      if (wave_any(answer && inner_tie)) {
-        // ids of every run of equal keys into the order of their labels (the filter's LDS is the buffer:
-        // the query is over)
-        uint32_t* tmp = reinterpret_cast<uint32_t*>(sets);
-        const bool on = answer && inner_tie;
-        if (on)
-          for (int e = hl; e < T; e += 32) tmp[e] = nbuf[e];
-        wave_sync();
-        if (on)
-          for (int e = hl; e < T; e += 32) {
-            const float k = dbuf[e];
-            const uint32_t me = tmp[e];
-            const uint64_t ml = ix.labels ? ix.labels[me] : (uint64_t)me;
-            int rank = e;
-            for (int f = e - 1; f >= 0 && dbuf[f] == k; --f) {
-              const uint32_t o = tmp[f];
-              rank -= (ix.labels ? ix.labels[o] : (uint64_t)o) > ml ? 1 : 0;
-            }
-            for (int f = e + 1; f < T && dbuf[f] == k; ++f) {
-              const uint32_t o = tmp[f];
-              rank += (ix.labels ? ix.labels[o] : (uint64_t)o) < ml ? 1 : 0;
-            }
-            nbuf[rank] = me;
-          }
-        wave_sync();
-      }
-      if (!a.hnswlib_dist) {
-        pair_dist<DT, QR, true>(ix, qv, nbuf, answer ? T : 0, dbuf, lane);
-        wave_sync();
-      }
-      if (answer) {
-        for (int r = hl; r < a.k; r += 32) {
-          int out_id = -1;
-          float out_d = INFINITY;
-          if (r < T) {
-            const uint32_t id = nbuf[r];
-            out_id = ix.labels ? (int)ix.labels[id] : (int)id;
-            out_d = dbuf[r];
-          }
-          a.nns[(size_t)qi * a.k + r] = out_id;
-          a.dists[(size_t)qi * a.k + r] = out_d;
-        }
-        if (hl == 0) {
-          a.found[qi] = T;
-          if (a.stats) {
-            a.stats[(size_t)qi * 4 + 0] = n_dist;
-            a.stats[(size_t)qi * 4 + 1] = n_hops;
-            a.stats[(size_t)qi * 4 + 2] = n_dist_upper;
-            a.stats[(size_t)qi * 4 + 3] = n_sweeps;
-          }
-        }
-      }
-      // results and list entry first, then the count the literal pass watches
-      __threadfence();
-      if (ending && hl == 0) atomicAdd(a.done, 1);
-      if (ending) {
-        phase = PP_NEED;
-        if (hl == 0) nbuf[0] = 0u;
-      }
-      wave_sync();
-    }
   }
 }
 
@@ -982,9 +639,43 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
       if (lane == 0) s.nbuf[0] = cur;
       wave_sync();
       bool ambiguous = false;
-      search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous,
-                                    tmeta.x >= 0 ? a.trail + (size_t)tmeta.x * a.trail_cap : nullptr, tmeta.y,
-                                    tmeta.x >= 0 ? tmeta.z : 0, tmeta.w);
+      // A trail that covers a whole search and sets no stretch apart IS hnswlib's sequence of accepted entries
+      // (after the entry point): what is open is only which of several equal keys at the cut its result heap
+      // keeps, so that heap alone is replayed — no queue, no set, no rows.
+      const uint4* trail = tmeta.x >= 0 ? a.trail + (size_t)tmeta.x * a.trail_cap : nullptr;
+      bool heap_only = trail != nullptr && tmeta.z < 0;
+      if (heap_only) {
+        bool marker = false;
+        for (int i = lane; i < tmeta.y; i += 64) marker = marker || trail[i].x >= kTrailBack;
+        heap_only = __ballot(marker) == 0ull;
+      }
+      const int trail_hops = tmeta.z < 0 ? -tmeta.z : tmeta.z;
+      if (heap_only) {
+        LdsHeap top{s.top};
+        int size = 0;
+        HeapEnt seed;
+        seed.key = dcur;
+        seed.id = cur;
+        coop_push<false>(top, size, seed, lane);
+        for (int base = 0; base < tmeta.y; base += 64) {
+          const int cnt = tmeta.y - base < 64 ? tmeta.y - base : 64;
+          const uint4 r = trail[base + (lane < cnt ? lane : 0)];   // 64 records per fetch, handed out lane by lane
+          for (int j = 0; j < cnt; ++j) {
+            HeapEnt e;
+            e.key = __builtin_bit_cast(float, __builtin_amdgcn_readlane((int)r.z, j));
+            e.id = (uint32_t)__builtin_amdgcn_readlane((int)r.y, j);
+            coop_push<false>(top, size, e, lane);
+            if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
+          }
+        }
+        st.top_size = size;
+        st.n_hops = trail_hops;
+        st.n_dist = tmeta.w;
+        literal = true;
+        T = 0;  // (set below, once the heap is down to k entries)
+      } else {
+      search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous, trail, tmeta.y,
+                                    trail != nullptr ? trail_hops : 0, tmeta.w);
       T = st.top_size < a.k ? st.top_size : a.k;
       // The first T entries of the set (equal keys among them in label order) are hnswlib's
       // answer unless equal keys sit across the cut, or the whole set is returned after an
@@ -1009,6 +700,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
           if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
         }
         st.top_size = size;
+      }
       }
     } else {
     vcache_reset(s, lane);

@@ -10,7 +10,10 @@
  *   - functions returning int: 0 = success, non-zero = failure; the message is
  *     available from cuhnsw_last_error(engine) (the reference throws
  *     std::runtime_error instead, cpp/include/cuda_base_kernels.cuh:30-37).
- *   - an engine is not thread-safe; calls are synchronous.
+ *   - calls are synchronous.  Every call on an engine takes that engine's lock, so calls from several
+ *     threads on ONE engine run one after the other (the reference relies on Python's GIL for that,
+ *     cuhnsw/bindings.cc has no gil_scoped_release); different engines run side by side.
+ *     cuhnsw_last_error reports the last failed call on the engine, whichever thread made it.
  *   - distances: dist_type "dot" -> -<q,x>, "l2" -> squared L2
  *     (cpp/include/cuda_dist_kernels.cuh:112-124).  Candidates are *ordered* by
  *     hnswlib's key (1 - <q,x> for "dot") so that ids equal hnswlib's.
@@ -87,8 +90,9 @@ int cuhnsw_search_knn(cuhnsw_engine* e, const float* qdata, int num_queries, int
 int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
                              int* d_nns, float* d_distances, int* d_found_cnt, int* d_stats, float* kernel_ms);
 
-/* The same search for callers that must not allocate device memory (code recorded into a HIP graph,
- * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+/* The same search for callers that must not allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc, code that runs beside a stream capture).  The call itself is synchronous and reads its
+ * status back: it cannot be recorded into a HIP graph.  It has no counterpart in the reference, whose
  * SearchGraph allocates on every call (cpp/src/cuhnsw_build.cu:238-249).  Neither this call nor
  * anything it runs calls hipMalloc, hipFree or a memset: the scratch memory of its kernels (control
  * words, the list of queries handed from the first pass to the literal pass, the literal wavefronts'
@@ -98,9 +102,10 @@ int cuhnsw_search_knn_device(cuhnsw_engine* e, const float* d_qdata, int num_que
  * literal search that outgrows its share of the array (4096 queued candidates beyond its LDS queue, 8192
  * accepted entries) makes the call fail; cuhnsw_search_knn_device answers such a batch.  The first pass
  * always runs (tunables fast_path, concurrent_literal and lean_literal do not apply) and the literal pass
- * follows it on the same stream.  All calls on one GPU share the array: calls that overlap in time on one
- * GPU — from several engines or threads — race; serialise them.  Same results as
- * cuhnsw_search_knn_device, bit for bit. */
+ * follows it on the same stream.  All calls on one GPU share the array, so only one of them runs at a time
+ * on a GPU: a call that finds another one under way — from another engine or thread of the process —
+ * fails at once with a message instead of racing with it.  Same results as cuhnsw_search_knn_device, bit
+ * for bit. */
 int cuhnsw_search_knn_device_noalloc(cuhnsw_engine* e, const float* d_qdata, int num_queries, int topk, int ef_search,
                                      int* d_nns, float* d_distances, int* d_found_cnt, float* kernel_ms);
 
@@ -150,6 +155,17 @@ int cuhnsw_last_search_repeats(cuhnsw_engine* e);
  * from them up to the point where the two searches may part (tunable "trails"; no counterpart in the
  * reference) */
 int cuhnsw_last_search_trails(cuhnsw_engine* e);
+/* 1 if the last search ran its literal pass beside the first pass (on a second stream), 0 if after it.
+ * No counterpart in the reference (one kernel, one stream, cpp/src/cuhnsw_build.cu:254-275). */
+int cuhnsw_last_search_side_by_side(cuhnsw_engine* e);
+/* How often, since the index became resident, a literal wavefront's bounded wait for the first pass ran out
+ * (the two streams were not running side by side: a profiler that serialises kernels, a saturated device).
+ * Each time the batch is answered after its first pass instead, and the next 8 searches run their passes one
+ * after the other before the side-by-side schedule is tried again; the "concurrent_literal" tunable itself
+ * is never changed by the engine. */
+int cuhnsw_literal_fallbacks(cuhnsw_engine* e);
+/* 1 unless the trail buffers (tunable "trails") could not be allocated; searches then go on without trails */
+int cuhnsw_trails_available(cuhnsw_engine* e);
 /* tuning knobs that are not part of the reference's option table:
  *   "build_batch"   largest number of nodes inserted per batch (default 0 = by the size of the graph: a quarter
  *                   of the nodes already in, at most 16384; beyond 524288 nodes a thirty-second, at most 65536)
@@ -172,10 +188,6 @@ int cuhnsw_last_search_trails(cuhnsw_engine* e);
  *                   first and takes its queries by descending distance of their level-0 entry point (the longest
  *                   searches first: a launch ends when its last query does); 2 = from more than one round on;
  *                   0 = in the caller's order.  Same answers and counters either way.
- *   "pair_path"     2 = the first pass runs two queries per wavefront (32 lanes each) wherever the shapes allow
- *                   it: ef_search up to 128, vectors of at most 128 dimensions, max_m and max_m0 at most 32;
- *                   0 = always one query per wavefront; 1 (default) = whichever is the faster one, which at
- *                   present is one query per wavefront in every measured shape.  Same results either way.
  *   "first_pass_waves" wavefronts per CU of the first pass (0 = as many as fit, the default)
  *   "concurrent_literal" 1 = the literal pass runs beside the first pass on a second stream
  *                   (default), 0 = after it
@@ -184,7 +196,7 @@ int cuhnsw_last_search_trails(cuhnsw_engine* e);
  *   "literal_spin_limit" polls one of its wavefronts may spend waiting for the first pass before
  *                   it leaves and the host answers the remaining queries afterwards (-1 = no bound in
  *                   polls: it leaves when the first pass has not started within 2 ms or stalls for
- *                   100 ms, and the engine then runs the passes one after the other from then on)
+ *                   100 ms; see cuhnsw_literal_fallbacks for what follows)
  *   "build_counters" 1 = count the work of the next builds on the device (cuhnsw_last_build_counters)
  *   "keep_link_keys" 1 = keep the keys stored with the level-0 links after build_graph for
  *                   cuhnsw_debug_link_keys0
@@ -195,7 +207,9 @@ int cuhnsw_last_search_trails(cuhnsw_engine* e);
  *                   certainly hnswlib's; the literal pass starts a handed-over query from there instead of from
  *                   the entry point (cuhnsw_last_search_trails counts them).  Needs the literal pass on the tag
  *                   filter (lean_literal), one query per wavefront, link rows under 64 ids, vectors of up to
- *                   128 elements; 266 MB of device memory for 2048 accepted entries per query at work.  Keeping
+ *                   128 elements; 270 MB of device memory for 2048 accepted entries per query at work,
+ *                   allocated when the index becomes resident (build_graph, load_index) — if that memory is
+ *                   not there, searches go on without trails (cuhnsw_trails_available).  Keeping
  *                   the trail costs the first pass 2 to 3 %: 1 (default) = for batches of up to two rounds of
  *                   wavefronts, which wait for their last hand-over; 2 = for every batch; 0 = off.
  *   "trail_cap"     accepted entries a trail holds (default 2048; a search that accepts more leaves none)

@@ -111,40 +111,6 @@ def test_search_parity_on_oracle_built_index(oracle, tmp_path, name, n, d, dist,
     _check_parity(oracle, ix, e, q, k, ef)
 
 
-@pytest.mark.parametrize("name,n,d,dist,max_m,max_m0,kind", [CASES[0], CASES[1], CASES[2], CASES[5], CASES[6]],
-                         ids=[CASES[i][0] for i in (0, 1, 2, 5, 6)])
-def test_two_queries_per_wavefront_equal_one_per_wavefront(oracle, tmp_path, name, n, d, dist, max_m, max_m0, kind):
-  """Small ef_search (up to 128): the first pass runs two queries per wavefront, each on half of its lanes.
-  Same answers, same counters and the same queries handed to the literal pass as with one query per
-  wavefront, and both equal to the oracle — odd and even batch sizes, a batch of one, tie-heavy data."""
-  x = _data(kind, n, d, 1)
-  q = _data(kind, 333, d, 2)
-  mult = 1.0 / np.log(max_m)
-  ix = oracle.OracleIndex(dist).build(x, _levels(n, mult, 3), max_m, max_m0, 60, mult)
-  p = str(tmp_path / "i.idx")
-  ix.save(p)
-  e = _engine(tmp_path, dist_type=dist, max_m=max_m, max_m0=max_m0)
-  e.load_index(p)
-  e.set_tunable("fast_path", 2)
-  for nq, k, ef in ((333, 10, 64), (332, 1, 1), (1, 10, 40), (2, 10, 128), (333, 100, 100), (333, 128, 128), (77, 5, 17)):
-    o_ids, o_d, o_f, o_cnt = ix.search(q[:nq], k, ef, counters=True)
-    got = {}
-    for pair in (1, 0):
-      e.set_tunable("pair_path", 2 if pair else 0)   # 2: the pair kernel wherever the shapes allow it
-      got[pair] = _device_search(e, q[:nq], k, ef) + (e.last_search_repeats,)
-      g_ids, g_d, g_f, stats, _ = got[pair]
-      assert (g_f == o_f).all()
-      for r in range(nq):
-        f = o_f[r]
-        assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d pair_path %d k %d ef %d" % (r, pair, k, ef)
-        assert (g_d[r, :f] == o_d[r, :f]).all()
-      assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
-    # evaluation counts too, and the same queries handed over (unless the engine has stopped trying the
-    # first pass on this index because most of its queries tie, which makes the second run literal-only)
-    assert (got[0][3] == got[1][3]).all() and (got[0][4] == got[1][4] or got[0][4] == 0)
-  e.set_tunable("pair_path", 1)
-
-
 @pytest.mark.parametrize("kind,d,dist,max_m,half", [
     ("gauss", 50, "dot", 8, False), ("int", 24, "l2", 8, False),
     ("gauss_raw", 100, "l2", 20, False),   # two register chunks per lane; upper-level rows longer than 16 ids
@@ -166,8 +132,7 @@ def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, k
   if half:
     e.set_tunable("fp16_storage", 1)
   e.load_index(p)
-  for pair, ef in ((0, 150), (2, 64)):   # one query per wavefront; two (which start level 0 at the stored entry too)
-    e.set_tunable("pair_path", pair)
+  for ef in (150, 64):
     got = {}
     for order in (2, 0):          # 2: in order whenever the batch is more than one round of wavefronts
       e.set_tunable("query_order", order)
@@ -184,7 +149,6 @@ def test_longest_queries_first_changes_nothing_but_the_order(oracle, tmp_path, k
     assert (g_f[:1500] == o_f).all() and (g_ids[:1500] == o_ids).all() and (g_d[:1500] == o_d).all()
     assert (stats[:1500, 1:] == o_cnt[:, 1:4]).all()
   e.set_tunable("query_order", 1)
-  e.set_tunable("pair_path", 1)
 
 
 def test_tight_rows_layout_and_gather_probe(oracle, tmp_path):
@@ -324,6 +288,58 @@ def test_literal_pass_schedules_on_tie_heavy_data(oracle, tmp_path):
     _check_parity(oracle, ix, e, q, 100, 100)
 
 
+def test_fallback_schedule_is_temporary_and_trails_are_optional(oracle, tmp_path):
+  """A literal wavefront whose wait runs out (forced from the host: a bound of zero polls) makes the engine answer
+  the batch after its first pass and run the next 8 searches one pass after the other; then the side-by-side
+  schedule is back, the caller's concurrent_literal setting untouched throughout.  A new index forgets all of it.
+  And trail buffers that cannot be allocated (a trail_cap of 2^30 entries) switch the trails off, not the search."""
+  n, d = 5000, 16
+  x = integer_vectors(n, d, seed=21, hi=30)
+  q = integer_vectors(150, d, seed=22, hi=30)
+  mult = 1 / np.log(8)
+  ix = oracle.OracleIndex("l2").build(x, _levels(n, mult, 23), 8, 16, 60, mult)
+  p = str(tmp_path / "t.idx")
+  ix.save(p)
+  o_ids, o_d, o_f = ix.search(q, 10, 100)
+  e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
+  e.load_index(p)
+  assert e.trails_available and e.literal_fallbacks == 0
+  e.set_tunable("fast_path", 2)
+  e.set_tunable("lean_literal", 2)
+
+  def search():
+    g_ids, g_d, g_f = e.search_knn(q, 10, 100)
+    assert (g_f == o_f).all() and (g_ids == o_ids).all() and (g_d == o_d).all()
+    assert e.last_search_repeats > 0
+
+  search()
+  assert e.last_search_side_by_side and e.last_search_trails > 0
+  e.set_tunable("literal_spin_limit", 0)
+  search()                                         # beside the first pass, every waiting wavefront gives up at once
+  assert e.last_search_side_by_side and e.literal_fallbacks == 1
+  e.set_tunable("literal_spin_limit", -1)
+  for _ in range(8):
+    search()
+    assert not e.last_search_side_by_side
+  search()
+  assert e.last_search_side_by_side and e.literal_fallbacks == 1
+  e.set_tunable("literal_spin_limit", 0)
+  search()
+  assert e.literal_fallbacks == 2
+  e.set_tunable("literal_spin_limit", -1)
+  e.load_index(p)                                  # another index: nothing of that is carried over
+  assert e.literal_fallbacks == 0
+  search()
+  assert e.last_search_side_by_side
+  # trails that cannot be allocated
+  e.set_tunable("trail_cap", 1 << 30)
+  search()
+  assert not e.trails_available and e.last_search_trails == 0
+  e.set_tunable("trail_cap", 2048)
+  search()
+  assert e.trails_available and e.last_search_trails > 0
+
+
 @pytest.mark.parametrize("d,hi", [(16, 30), (12, 60), (80, 6)], ids=["many_ties", "fewer_ties", "two_chunks_per_lane"])
 def test_handed_over_queries_start_from_the_first_pass_trail(oracle, tmp_path, d, hi):
   """The first pass leaves the entries it accepted, hop by hop, and the literal pass (on the tag filter) replays
@@ -341,7 +357,6 @@ def test_handed_over_queries_start_from_the_first_pass_trail(oracle, tmp_path, d
   e.load_index(p)
   e.set_tunable("fast_path", 2)
   e.set_tunable("lean_literal", 2)
-  e.set_tunable("pair_path", 0)
   for k, ef in ((10, 100), (100, 100), (10, 300)):
     o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
     # (eight wavefronts: each answers some thirty queries and needs a spare buffer after every hand-over; trails = 2:
@@ -367,7 +382,7 @@ def test_handed_over_queries_start_from_the_first_pass_trail(oracle, tmp_path, d
         assert trails <= handed
       else:
         assert trails == 0
-  for key, value in (("trails", 1), ("trail_cap", 2048), ("trail_spares", 1024), ("concurrent_literal", 1), ("pair_path", 1),
+  for key, value in (("trails", 1), ("trail_cap", 2048), ("trail_spares", 1024), ("concurrent_literal", 1),
                      ("search_slots", 0)):
     e.set_tunable(key, value)
 
