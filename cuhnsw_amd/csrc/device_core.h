@@ -1184,7 +1184,7 @@ template <int DT, int QR, int NS>
 __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec<QR>& qv, int ef, Scratch& s, SearchState& st,
                                                   Frontier<NS>& fr, int n_seed, int lane, bool* ambiguous,
                                                   const uint4* trail = nullptr, int trail_n = 0, int trail_hops = 0,
-                                                  int trail_n_dist = 0) {
+                                                  int trail_n_dist = 0, int stop_marker = -1, int* rest_from = nullptr) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
   const int S = row_stride(ix, 0);
@@ -1267,6 +1267,12 @@ __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec
         if (trail_at >= trail_n || kind < kTrailBack || at_hop != (uint32_t)st.n_hops) break;
         own_stretch = kind == kTrailOwn;
         trail_at += 1;
+      }
+      // (stop_marker >= 0: the trail covers the whole search and this is the index of its last marker.  Once past
+      // it, every further accepted entry is on the trail: the caller needs no more of this search.)
+      if (stop_marker >= 0 && !own_stretch && trail_at > stop_marker) {
+        *rest_from = trail_at;
+        break;
       }
       if (!own_stretch) {
         // this hop's records: a run from trail_at on (at most one link row's worth: under 64)

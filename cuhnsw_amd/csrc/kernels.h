@@ -639,25 +639,42 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
       if (lane == 0) s.nbuf[0] = cur;
       wave_sync();
       bool ambiguous = false;
-      // A trail that covers a whole search and sets no stretch apart IS hnswlib's sequence of accepted entries
-      // (after the entry point): what is open is only which of several equal keys at the cut its result heap
-      // keeps, so that heap alone is replayed — no queue, no set, no rows.
+      // A trail that covers a whole search (the first pass went all the way: only the cut at k is open) IS
+      // hnswlib's sequence of accepted entries wherever it sets no stretch apart.  From its last marker on
+      // nothing but the result heap needs replaying: the search below stops there (with no marker at all it
+      // is not even started), and the heap is fed from the log of what the search accepted so far and then
+      // from the rest of the trail — no queue, no set, no rows.
       const uint4* trail = tmeta.x >= 0 ? a.trail + (size_t)tmeta.x * a.trail_cap : nullptr;
-      bool heap_only = trail != nullptr && tmeta.z < 0;
-      if (heap_only) {
-        bool marker = false;
-        for (int i = lane; i < tmeta.y; i += 64) marker = marker || trail[i].x >= kTrailBack;
-        heap_only = __ballot(marker) == 0ull;
-      }
+      const bool whole = trail != nullptr && tmeta.z < 0;
       const int trail_hops = tmeta.z < 0 ? -tmeta.z : tmeta.z;
-      if (heap_only) {
+      int last_marker = -1;
+      if (whole) {
+        for (int base = 0; base < tmeta.y; base += 64) {
+          const int i = base + lane;
+          const unsigned long long m = __ballot(i < tmeta.y && trail[i < tmeta.y ? i : 0].x >= kTrailBack);
+          if (m != 0ull) last_marker = base + 63 - __builtin_clzll(m);
+        }
+      }
+      int rest_from = (whole && last_marker < 0) ? 0 : -1;  // >= 0: the trail's records from here on are the rest of the accepted sequence
+      if (rest_from < 0)
+        search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous, trail, tmeta.y,
+                                      trail != nullptr ? trail_hops : 0, tmeta.w, whole ? last_marker : -1, &rest_from);
+      if (rest_from >= 0 && !st.fail) {
+        __threadfence_block();
         LdsHeap top{s.top};
         int size = 0;
-        HeapEnt seed;
-        seed.key = dcur;
-        seed.id = cur;
-        coop_push<false>(top, size, seed, lane);
-        for (int base = 0; base < tmeta.y; base += 64) {
+        if (st.n_acc == 0) {  // (no search was made: the entry point is the first accepted entry)
+          HeapEnt seed;
+          seed.key = dcur;
+          seed.id = cur;
+          coop_push<false>(top, size, seed, lane);
+        }
+        for (int i = 0; i < st.n_acc; ++i) {
+          const HeapEnt e = uniform_ent(s.log[i]);
+          coop_push<false>(top, size, e, lane);
+          if (size > a.ef) coop_pop<false>(top, size, s.tree, lane);
+        }
+        for (int base = rest_from; base < tmeta.y; base += 64) {
           const int cnt = tmeta.y - base < 64 ? tmeta.y - base : 64;
           const uint4 r = trail[base + (lane < cnt ? lane : 0)];   // 64 records per fetch, handed out lane by lane
           for (int j = 0; j < cnt; ++j) {
@@ -670,12 +687,10 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
         }
         st.top_size = size;
         st.n_hops = trail_hops;
-        st.n_dist = tmeta.w;
+        if (st.n_acc == 0) st.n_dist = tmeta.w;
         literal = true;
         T = 0;  // (set below, once the heap is down to k entries)
       } else {
-      search_level_lean<DT, QR, NS>(ix, qv, a.ef, s, st, fr, 1, lane, &ambiguous, trail, tmeta.y,
-                                    trail != nullptr ? trail_hops : 0, tmeta.w);
       T = st.top_size < a.k ? st.top_size : a.k;
       // The first T entries of the set (equal keys among them in label order) are hnswlib's
       // answer unless equal keys sit across the cut, or the whole set is returned after an
