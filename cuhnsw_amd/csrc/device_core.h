@@ -455,7 +455,9 @@ __device__ __forceinline__ void undo_visited(Scratch& s, SearchState& st, int la
   } else {
     for (int w = lane; w < s.bitmap_words; w += 64) s.bitmap[w] = 0u;
   }
-  __threadfence();
+  // (the bitmap belongs to this wavefront alone: its clearing stores only have to be done before its next
+  // atomics are issued.  An agent-scope fence here would write the L2 back and invalidate the L1 once per query.)
+  __threadfence_block();
   st.undo_cnt = 0;
 }
 
@@ -920,6 +922,76 @@ __device__ __forceinline__ void trail_stop(Trail& tr, int hops, int n_dist) {
   }
 }
 
+// One phase of the tie-free loop of search_level_fast (below).  Nine searches in ten never hold two equal keys in
+// their set; until the first such pair turns up the search runs here, with none of the bookkeeping that equal keys
+// need.  FULL = false: while the set fills (the bound is the largest key accepted so far, every offer is accepted);
+// FULL = true: the set holds ef entries (the bound is its last key, an accepted offer pushes one out) — two
+// instantiations, so that the hot one carries neither the fill test nor the running maximum.  TRAILS: the hop's
+// accepted entries go on the search's trail (a kernel instance of its own: a pass that keeps no trails pays
+// nothing for them).  Returns 0: no waiting entry is left, the search is over; 1: an
+// offer met an equal key of another node (resume_at = which offer of the list in s.nbuf / s.dbuf); 2 (FULL = false
+// only): the set is full now, the other phase goes on.  n = ids waiting in s.nbuf on entry.
+template <int DT, int QR, int NS, bool FULL, bool TRAILS>
+__device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, int S, Scratch& s,
+                                              SearchState& st, Frontier<NS>& fr, int& n, int& hop_cid, int& resume_at,
+                                              unsigned long long& accepted, Trail& tr, int lane) {
+  constexpr int N = NS > 0 ? NS : 1;
+  while (true) {
+    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    st.n_dist += n;
+    wave_sync();
+    // (unconditional LDS reads at a clamped index, then a select: no exec-mask branches)
+    const int last = n > 0 ? n - 1 : 0;
+    const int at = lane < last ? lane : last;
+    const float got_key = s.dbuf[at];
+    const uint32_t my_id = s.nbuf[at];
+    const float my_key = lane < n ? got_key : INFINITY;
+    unsigned long long todo = FULL ? __ballot(st.lower > my_key) : __ballot(lane < n);
+    while (todo != 0ull) {
+      const int j = __builtin_ctzll(todo);
+      todo &= todo - 1ull;
+      const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+      const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+      if (FULL ? st.lower > key : (st.n_acc < ef || st.lower > key)) {
+        bool eq = false;
+#pragma unroll
+        for (int t = 0; t < N; ++t) eq = eq || fr.k[t] == key;
+        if (__ballot(eq) == 0ull) {
+          frontier_insert_distinct<NS>(fr, key, id);
+          accepted |= 1ull << j;
+          st.n_acc = st.n_acc + 1;
+          if (!FULL && st.n_acc < ef) {
+            st.maxkey = uni(fmaxf(st.maxkey, key));
+            st.lower = st.maxkey;
+          } else {
+            st.lower = frontier_max<NS>(fr);  // hnswlib's lowerBound
+          }
+        } else {
+          bool same = false;
+#pragma unroll
+          for (int t = 0; t < N; ++t) same = same || (fr.k[t] == key && (fr.v[t] & ~kExpanded) == id);
+          if (__ballot(same) == 0ull) {
+            resume_at = j;  // an equal key of another node: the rules for equal keys apply from this offer on
+            todo = 0ull;
+          }
+          // (else: a node met again after the visited filter forgot it; it is in the set already)
+        }
+      }
+    }
+    if (resume_at >= 0) return 1;
+    if (TRAILS) trail_hop(tr, accepted, hop_cid, st.n_hops, my_id, my_key, lane);
+    accepted = 0ull;
+    const int cid = frontier_take<NS>(fr, lane, false);
+    if (cid < 0) return 0;
+    hop_cid = cid;
+    st.n_hops += 1;
+    wave_sync();
+    n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
+    wave_sync();
+    if (!FULL && st.n_acc >= ef) return 2;
+  }
+}
+
 // Best-first search of one level on the sorted set (needs the LDS tag filter).  On entry
 // s.nbuf[0..n_seed) holds the seeds, already entered into the filter.  Returns 0: fr holds the
 // result (st.top_size entries, ascending), all keys were distinct; 2: the same, but equal keys
@@ -956,7 +1028,7 @@ __device__ __forceinline__ void trail_stop(Trail& tr, int hops, int n_dist) {
 // far: expand the farthest waiting entry instead of the closest (the reference's
 // reverse_cand); that is no hnswlib search any more, equal keys simply keep their order of
 // arrival and nothing is ever given up.  BUILD likewise never gives up.
-template <int DT, int QR, int NS, bool BUILD>
+template <int DT, int QR, int NS, bool BUILD, bool TRAILS = false>
 __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
                                                   SearchState& st, Frontier<NS>& fr, int n_seed, int lane,
                                                   bool far = false, bool whole_set = false, Trail* trail = nullptr) {
@@ -976,68 +1048,15 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   float group_edge = INFINITY;        // closest key turned away or evicted while the group is expanded
   float ek_min = INFINITY;            // smallest key at which an eviction had equal largest keys to choose from
   bool gave_up = false;
-  // Nine searches in ten never see two equal keys in their set.  Until the first such pair turns up the
-  // search runs in a loop that carries none of the bookkeeping above — same decisions, half the
-  // instructions per accepted candidate — and only then moves on to the general loop below, at the very
-  // offer that met the equal key (resume_at).
+  // Until two equal keys meet in the set the search runs in tie_free_phase — same decisions, half the
+  // instructions per accepted candidate — and only then moves on to the general loop below, at the very offer
+  // that met the equal key (resume_at).
   int resume_at = -1;
   if (exact && S <= 64) {
-    bool finished = false;
-    while (true) {
-      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
-      st.n_dist += n;
-      wave_sync();
-      const int at = lane < n ? lane : 0;
-      const float my_key = lane < n ? s.dbuf[at] : INFINITY;
-      const uint32_t my_id = s.nbuf[at];
-      unsigned long long todo = __ballot(lane < n && (st.n_acc < ef || st.lower > my_key));
-      while (todo != 0ull) {
-        const int j = __builtin_ctzll(todo);
-        todo &= todo - 1ull;
-        const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
-        const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
-        if (st.n_acc < ef || st.lower > key) {
-          bool eq = false;
-#pragma unroll
-          for (int t = 0; t < (NS > 0 ? NS : 1); ++t) eq = eq || fr.k[t] == key;
-          if (__ballot(eq) == 0ull) {
-            frontier_insert_distinct<NS>(fr, key, id);
-            accepted |= 1ull << j;
-            st.n_acc = st.n_acc + 1;
-            if (st.n_acc < ef) {
-              st.maxkey = uni(fmaxf(st.maxkey, key));
-              st.lower = st.maxkey;
-            } else {
-              st.lower = frontier_max<NS>(fr);  // hnswlib's lowerBound
-            }
-          } else {
-            bool same = false;
-#pragma unroll
-            for (int t = 0; t < (NS > 0 ? NS : 1); ++t) same = same || (fr.k[t] == key && (fr.v[t] & ~kExpanded) == id);
-            if (__ballot(same) == 0ull) {
-              resume_at = j;  // an equal key of another node: the rules for equal keys apply from this offer on
-              todo = 0ull;
-            }
-            // (else: a node met again after the visited filter forgot it; it is in the set already)
-          }
-        }
-      }
-      if (resume_at >= 0) break;
-      trail_hop(tr, accepted, hop_cid, st.n_hops, my_id, my_key, lane);
-      accepted = 0ull;
-      st.top_size = st.n_acc < ef ? st.n_acc : ef;
-      const int cid = frontier_take<NS>(fr, lane, false);
-      if (cid < 0) {
-        finished = true;
-        break;
-      }
-      hop_cid = cid;
-      st.n_hops += 1;
-      wave_sync();
-      n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
-      wave_sync();
-    }
-    if (finished) {
+    int how = st.n_acc >= ef ? 2 : tie_free_phase<DT, QR, NS, false, TRAILS>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, lane);
+    if (how == 2) how = tie_free_phase<DT, QR, NS, true, TRAILS>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, lane);
+    st.top_size = st.n_acc < ef ? st.n_acc : ef;
+    if (how == 0) {
       trail_stop(tr, st.n_hops, st.n_dist);
       return 0;
     }

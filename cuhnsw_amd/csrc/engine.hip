@@ -560,7 +560,7 @@ class Engine {
         (a.fast_path > 1 || a.nq > lit_slots || (a.lean && a.nq > 1))) {  // (reverse_cand: fast_path is 2)
       d_redo.reserve((size_t)a.nq);
       a.redo = d_redo.p;
-      auto fast_kernel = search_fast_kernel<DT, QR, NS>;
+      auto fast_kernel = search_fast_kernel<DT, QR, NS, false>;
       auto fast_lds = [&](int bits) -> size_t { return plan_fast_lds(QR, ix.Dp, a.lcap, bits).total; };
       auto fast_slots = [&](int bits) -> int { return resident_slots(fast_kernel, fast_lds(bits)); };
       // the filter must not be what limits the wavefronts per CU: half the filter repeats more
@@ -683,7 +683,12 @@ class Engine {
                            a.nq, d_order_hist.p, d_order.p);
         HIP_CHECK(hipGetLastError());
       }
-      hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
+      if constexpr (QR == 1 || QR == 2) {
+        if (keep_trails) hipLaunchKernelGGL((search_fast_kernel<DT, QR, NS, true>), dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
+        else hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
+      } else {
+        hipLaunchKernelGGL(fast_kernel, dim3(slots), dim3(64), fast_lds_bytes, stream, ix, a);
+      }
       HIP_CHECK(hipGetLastError());
       if (side) {
         HIP_CHECK(hipStreamWaitEvent(stream, ev_side1, 0));
@@ -759,7 +764,7 @@ class Engine {
       a.fast_path = 2;
       a.lean = a.fc_bits;  // literal searches keep the LDS filter and the sorted set with ids: no bitmap in HBM
       auto kernel = search_kernel<DT, QR, NS>;
-      auto fast_kernel = search_fast_kernel<DT, QR, NS>;
+      auto fast_kernel = search_fast_kernel<DT, QR, NS, false>;
       while (filter_entries <= 0 && a.fc_bits > 9) {  // (as in the allocating search: the filter must not cost occupancy)
         const int now = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits).total);
         const int with_half = resident_slots(fast_kernel, plan_fast_lds(QR, ix.Dp, a.lcap, a.fc_bits - 1).total);

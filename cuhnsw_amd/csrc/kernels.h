@@ -383,10 +383,10 @@ __global__ void __launch_bounds__(1024) order_scatter_kernel(const uint4* entry,
 // held to 72 registers, seven wavefronts per SIMD, at the price of up to five spilled registers;
 // eight wavefronts are no faster; with eight keys per lane it fits 96 registers, five wavefronts
 // per SIMD, without spilling; the other shapes would spill heavily)
-// With a.trail set the pass leaves trails for the literal pass (2 to 3 % more instructions: the host asks for
-// them in batches of a round or two of wavefronts, where a query handed over late is a good part of the
-// batch's time).
-template <int DT, int QR, int NS>
+// TRAILS: the pass leaves trails for the literal pass (a.trail set; 2 to 3 % more instructions: the host launches
+// this instance for batches of a round or two of wavefronts, where a query handed over late is a good part of the
+// batch's time, and the instance without the trail code otherwise).
+template <int DT, int QR, int NS, bool TRAILS>
 __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS == 8 ? 5 : 1)) : 1) search_fast_kernel(DevIndex ix, SearchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x;
@@ -399,7 +399,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
   s.dbuf = reinterpret_cast<float*>(smem + lp.dbuf);
   // tells a literal pass waiting beside this one that the two kernels do run at the same time
   if (blockIdx.x == 0 && lane == 0) __hip_atomic_store(a.done + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  int trail_buf = a.trail ? (int)blockIdx.x : -1;  // the buffer this wavefront's trails go to
+  int trail_buf = (TRAILS && a.trail) ? (int)blockIdx.x : -1;  // the buffer this wavefront's trails go to
 
   for (;;) {
     int qi = 0;
@@ -410,7 +410,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     qi = __builtin_amdgcn_readfirstlane(qi);
     if (qi >= a.nq) break;
     Trail tr;
-    if (trail_buf >= 0) {
+    if (TRAILS && trail_buf >= 0) {
       tr.rec = a.trail + (size_t)trail_buf * a.trail_cap;
       tr.cap = a.trail_cap;
       tr.on = true;
@@ -440,7 +440,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     wave_sync();
     // (the flag is made wavefront-uniform explicitly and both outcomes are plain branches)
     const int how =
-        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0, a.k >= a.ef, &tr));
+        __builtin_amdgcn_readfirstlane(search_level_fast<DT, QR, NS, false, TRAILS>(ix, qv, 0, a.ef, s, st, fr, 1, lane, a.reverse != 0, a.k >= a.ef, TRAILS ? &tr : nullptr));
     const int T0 = st.top_size < a.k ? st.top_size : a.k;
     // Equal keys across the cut at k: which of them stays is up to the result heap, which the
     // literal search reproduces.  Equal keys among the k best: the answer lists them by label.
@@ -450,7 +450,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
     const bool gave_up = how == 1 || cut_tie || (inner_tie && T0 > (1 << a.fc_bits));  // (the filter's LDS is the sort's buffer)
     if (gave_up) {
       // (the trail's records are written by many lanes: all of them out before lane 0 publishes the entry)
-      const bool with_trail = a.redo_trail && trail_buf >= 0 && tr.n > 0 && tr.hops > 0;
+      const bool with_trail = TRAILS && a.redo_trail && trail_buf >= 0 && tr.n > 0 && tr.hops > 0;
       // a search that went all the way (only the cut at k is open) and whose trail covers every hop: the literal
       // pass needs no search at all, only the result heap replayed from the trail (hops stored negative)
       const bool whole = how != 1 && tr.hops == st.n_hops;
@@ -498,9 +498,13 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
         }
       }
     }
-    // results and list entry first, then the count the literal pass watches
-    __threadfence();
-    if (lane == 0) atomicAdd(a.done, 1);
+    // The count the literal pass watches.  Only a query that was handed over has published something that pass
+    // reads (its list entry, its trail): there the count is raised with release order, after them; an answered
+    // query's results are the host's to read, after the kernel.
+    if (lane == 0) {
+      if (gave_up) __hip_atomic_fetch_add(a.done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_fetch_add(a.done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     wave_sync();
   }
 }
@@ -1002,8 +1006,10 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
         }
         if (deg > 0) cur = oid[0];  // closest selected neighbour: entry for the level below
         wave_sync();
-        undo_visited(s, st, lane);
-        wave_sync();
+        if (!sorted_set) {
+          undo_visited(s, st, lane);
+          wave_sync();
+        }
       }
       if (lane == 0 && st.fail) *a.status = 1;
       if (a.counters && lane == 0) {

@@ -29,12 +29,14 @@ DEVICE_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-ffp-contract=off
 
 # kernel instances the guard looks at: (template text, short name)
 FIRST_PASS = [
-    ("search_fast_kernel<DIST_DOT, 1, 5>(DevIndex, SearchArgs)", "search_fast_kernel<dot,1,5>"),
-    ("search_fast_kernel<DIST_L2, 1, 5>(DevIndex, SearchArgs)", "search_fast_kernel<l2,1,5>"),
-    ("search_fast_kernel<DIST_DOT, 2, 5>(DevIndex, SearchArgs)", "search_fast_kernel<dot,2,5>"),
-    ("search_fast_kernel<DIST_L2, 2, 5>(DevIndex, SearchArgs)", "search_fast_kernel<l2,2,5>"),
-    ("search_fast_kernel<DIST_DOT, 1, 2>(DevIndex, SearchArgs)", "search_fast_kernel<dot,1,2>"),
-    ("search_fast_kernel<DIST_DOT, 2, 8>(DevIndex, SearchArgs)", "search_fast_kernel<dot,2,8>"),
+    ("search_fast_kernel<DIST_DOT, 1, 5, false>(DevIndex, SearchArgs)", "search_fast_kernel<dot,1,5>"),
+    ("search_fast_kernel<DIST_DOT, 1, 5, true>(DevIndex, SearchArgs)", "search_fast_kernel<dot,1,5,trails>"),
+    ("search_fast_kernel<DIST_L2, 1, 5, false>(DevIndex, SearchArgs)", "search_fast_kernel<l2,1,5>"),
+    ("search_fast_kernel<DIST_DOT, 2, 5, false>(DevIndex, SearchArgs)", "search_fast_kernel<dot,2,5>"),
+    ("search_fast_kernel<DIST_L2, 2, 5, false>(DevIndex, SearchArgs)", "search_fast_kernel<l2,2,5>"),
+    ("search_fast_kernel<DIST_L2, 2, 5, true>(DevIndex, SearchArgs)", "search_fast_kernel<l2,2,5,trails>"),
+    ("search_fast_kernel<DIST_DOT, 1, 2, false>(DevIndex, SearchArgs)", "search_fast_kernel<dot,1,2>"),
+    ("search_fast_kernel<DIST_DOT, 2, 8, false>(DevIndex, SearchArgs)", "search_fast_kernel<dot,2,8>"),
 ]
 OTHERS = [
     ("search_kernel<DIST_DOT, 1, 5>(DevIndex, SearchArgs)", "search_kernel<dot,1,5>"),

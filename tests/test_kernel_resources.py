@@ -14,12 +14,14 @@ pytestmark = pytest.mark.skipif(shutil.which(kernel_report.HIPCC) is None, reaso
 
 # kernel -> (wavefronts per SIMD at least, scratch bytes per lane at most)
 LIMITS = {
-    "search_fast_kernel<dot,1,5>": (7, 60),
-    "search_fast_kernel<l2,1,5>": (7, 44),
-    "search_fast_kernel<dot,2,5>": (7, 72),
-    "search_fast_kernel<l2,2,5>": (7, 76),
-    "search_fast_kernel<dot,1,2>": (7, 20),
-    "search_fast_kernel<dot,2,8>": (5, 20),
+    "search_fast_kernel<dot,1,5>": (7, 36),
+    "search_fast_kernel<dot,1,5,trails>": (7, 56),
+    "search_fast_kernel<l2,1,5>": (7, 36),
+    "search_fast_kernel<dot,2,5>": (7, 36),
+    "search_fast_kernel<l2,2,5>": (7, 36),
+    "search_fast_kernel<l2,2,5,trails>": (7, 56),
+    "search_fast_kernel<dot,1,2>": (7, 0),
+    "search_fast_kernel<dot,2,8>": (5, 0),
 }
 
 
