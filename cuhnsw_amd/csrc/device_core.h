@@ -745,8 +745,9 @@ __device__ __forceinline__ int frontier_take(Frontier<NS>& f, int lane, bool far
     L = 63 - __builtin_clzll(mask);
   }
   const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)vf, L);
+  // (an id is in the set once: the entry that holds it is the one taken, whichever lane that is)
 #pragma unroll
-  for (int j = 0; j < N; ++j) f.v[j] = (lane == L && f.v[j] == id) ? (id | kExpanded) : f.v[j];
+  for (int j = 0; j < N; ++j) f.v[j] = f.v[j] == id ? (id | kExpanded) : f.v[j];
   return (int)id;
 }
 // key of the entry with this id (which is in the set)
@@ -840,16 +841,18 @@ __device__ __forceinline__ int visit_lossy(const uint32_t* row, int S, Scratch& 
   for (int base = 0; base < S; base += 64) {
     const uint32_t got = row[base + lane < S ? base + lane : 0];  // unconditional load, then a select
     const uint32_t id = (base + lane < S) ? got : kEmpty;
-    bool ask = id != kEmpty;
-    if (ask) {
-      const uint32_t slot = id & mask_bits;
-      const uint32_t tag = id >> set_bits;
-      const uint2 w = sets[slot];
-      ask = (w.x & 0xFFFFu) != tag && (w.x >> 16) != tag && (w.y & 0xFFFFu) != tag && (w.y >> 16) != tag;
-      if (ask) sets[slot] = filter_push(w, tag);
-    }
+    // (every lane looks its set up — an empty slot's id maps to some set and to a tag no set can hold — so that
+    // the only predicated part is the two LDS writes at the end)
+    const uint32_t slot = id & mask_bits;
+    const uint32_t tag = id >> set_bits;
+    const uint2 w = sets[slot];
+    const bool ask = (id != kEmpty) & ((w.x & 0xFFFFu) != tag) & ((w.x >> 16) != tag) & ((w.y & 0xFFFFu) != tag) &
+                     ((w.y >> 16) != tag);
     const unsigned long long mask = __ballot(ask);
-    if (ask) s.nbuf[n + __popcll(mask & ((1ull << lane) - 1ull))] = id;
+    if (ask) {
+      sets[slot] = filter_push(w, tag);
+      s.nbuf[n + __popcll(mask & ((1ull << lane) - 1ull))] = id;
+    }
     n += __popcll(mask);
   }
   return n;
@@ -958,7 +961,7 @@ __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>
         for (int t = 0; t < N; ++t) eq = eq || fr.k[t] == key;
         if (__ballot(eq) == 0ull) {
           frontier_insert_distinct<NS>(fr, key, id);
-          accepted |= 1ull << j;
+          if (TRAILS) accepted |= 1ull << j;
           st.n_acc = st.n_acc + 1;
           if (!FULL && st.n_acc < ef) {
             st.maxkey = uni(fmaxf(st.maxkey, key));
