@@ -98,6 +98,15 @@ __global__ void __launch_bounds__(128) fill_ints_kernel(int* p, int n, int value
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = value;
 }
+// Everything a two-pass search needs cleared, in one launch: the control words (0), the list the first pass
+// appends to (-1 = "no entry yet", which the literal wavefronts poll for) and, for a batch taken longest
+// first, the counters of the counting sort (0).
+__global__ void __launch_bounds__(256) prepare_search_kernel(int* ctl, int n_ctl, int* redo, int n_redo, int* hist, int n_hist) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_ctl) ctl[i] = 0;
+  if (i < n_redo) redo[i] = -1;
+  if (i < n_hist) hist[i] = 0;
+}
 
 template <typename T>
 struct DevBuf {
@@ -181,6 +190,7 @@ class Engine {
   int last_build_dropped = 0;  // reverse links of the last build that found no room in an inbox
   int keep_link_keys = 0;      // keep the keys stored with the level-0 links after a build (debugging aid)
   std::vector<float> link_keys0;  // N x max_m0, only with keep_link_keys
+  int newcomer_shortcut = 1;  // build: a link row that the selection rule produced is re-selected with the shortcut for newcomers
   int own_links0 = 0;  // links a new node selects for itself on level 0: 0 = max_m0 (as the reference), else min(value, max_m0); hnswlib uses max_m
   int spill_cap = 0;  // first size of the per-slot queue overflow area (0 = automatic); the accept log is twice that
   int visited_cache = 0;  // entries of the LDS visited cache: 0 = automatic, < 0 = none
@@ -528,7 +538,6 @@ class Engine {
     // caller asked for literal queues only, which also means exact evaluation counters
     // ...and unless the visited bitmaps of the wavefronts at work fit the L2 caches (32 MB) together:
     // there the bitmap's atomics are cheap and the literal search with them is the faster one
-    // (100 000 points, 1 000 queries: 1.10 ms against 1.33 ms; 1 M x 960, 1 000 queries: 8.8 against 5.9)
     const size_t bitmap_bytes = (size_t)std::min(num_cus * 24, a.nq) * ((host.N + 31) / 32) * 4;
     const bool want_lean = lean_literal == 1 ? bitmap_bytes > ((size_t)32 << 20) : lean_literal > 1;
     a.lean = (NS > 0 && fast_path != 0 && want_lean) ? auto_fc_bits(a.ef) : 0;
@@ -549,13 +558,12 @@ class Engine {
     int glob_cap = spill_cap > 0 ? spill_cap : std::max(4096, 8 * a.ef);
     int n_literal = a.nq;
     bool answered = false;
-    // A batch that fits the machine in one round of literal wavefronts is latency-bound: two
-    // passes would only add the second pass's latency to the first's — where the literal search has its exact
-    // bitmaps (100 000 points, 1 000 queries: 1.06 ms literal only; 0.75 ms through the first pass, but 1.76 when
-    // one query is handed over at its end).  Where the bitmaps do not fit the L2 and the literal search runs on the
-    // sorted set with the LDS filter, the first pass is the same search without the literal candidate queue, and
-    // the faster one even with a hand-over (1.18 M points, 2 000 queries: 1.73 against 2.36 ms; 1 M x 960, 1 000
-    // queries: 5.33 against 5.95 ms).
+    bool timed = false;  // ev1 has been recorded after the last kernel of this search
+    // A batch that fits the machine in one round of literal wavefronts is latency-bound: where the literal
+    // search has its exact bitmaps, two passes would only add the second pass's latency to the first's, and
+    // the literal pass answers alone.  Where the bitmaps do not fit the L2 (the literal search then runs on
+    // the sorted set with the LDS filter) the first pass is the same search without the literal candidate
+    // queue, and the faster choice even with a hand-over.
     if (NS > 0 && a.fast_path && a.fc_bits > 0 &&
         (a.fast_path > 1 || a.nq > lit_slots || (a.lean && a.nq > 1))) {  // (reverse_cand: fast_path is 2)
       d_redo.reserve((size_t)a.nq);
@@ -564,8 +572,7 @@ class Engine {
       auto fast_lds = [&](int bits) -> size_t { return plan_fast_lds(QR, ix.Dp, a.lcap, bits).total; };
       auto fast_slots = [&](int bits) -> int { return resident_slots(fast_kernel, fast_lds(bits)); };
       // the filter must not be what limits the wavefronts per CU: half the filter repeats more
-      // evaluations but is the faster choice wherever it buys occupancy (10 M x 96, ef = 512,
-      // five wavefronts per SIMD by registers: 46.8 ms with 8 KB of filter, 45.2 ms with 4 KB)
+      // evaluations but is the faster choice wherever it buys 15 % more wavefronts
       while (filter_entries <= 0 && a.fc_bits > 9) {
         const int now = fast_slots(a.fc_bits);
         const int with_half = fast_slots(a.fc_bits - 1);
@@ -577,10 +584,9 @@ class Engine {
       const bool side = concurrent_literal && sequential_left == 0 && max_slots_override <= 0;
       last_side_by_side = side ? 1 : 0;
       int side_slots = 0;
-      // few queries need the literal pass (0.4 % of the 1.18M-point set's): one wavefront per CU
-      // serves them without taking room from the first pass; two when the last search needed more
-      // (6.5 % on integer-valued 128-d data: 4.8 ms with one or two, 5.2 with four, 8.3 with eight —
-      // a literal wavefront's LDS is that of one and a half wavefronts of the first pass)
+      // few queries need the literal pass: one wavefront per CU serves them without taking room from
+      // the first pass; two when the last search handed over 2 % and more (a literal wavefront's LDS
+      // is that of one and a half wavefronts of the first pass, so more of them cost more than they serve)
       const int per_cu = side_per_cu > 0 ? side_per_cu : (last_repeat_share < 0.02 ? 1 : 2);
       if (side) {
         side_slots = std::min(num_cus * per_cu, a.nq);
@@ -593,24 +599,15 @@ class Engine {
       if (max_slots_override > 0) slots = max_slots_override;
       if (first_pass_waves > 0) slots = std::min(slots, first_pass_waves * num_cus);
       slots = std::max(1, std::min(slots, a.nq));
-      HIP_CHECK(hipMemsetAsync(d_ctl.p, 0, 128 * sizeof(int), stream));
-      HIP_CHECK(hipMemsetAsync(d_redo.p, 0xFF, (size_t)a.nq * sizeof(int), stream));
       // (every allocation before the literal pass is launched: growing a buffer frees the old one, and
       // hipFree waits for the device, on which that pass would be waiting for the first pass to start)
-      // (from one and a half rounds of wavefronts on — 1.18 M x 50, 40 000 queries: 8.25 -> 7.41 ms; eight draws of
-      // 12 000 queries, 1.7 rounds: 3.10 -> 2.85 ms on average; of 10 000, 1.4 rounds: 2.92 and 2.96 — the first
-      // pass alone gains, 2.8 -> 2.2 ms, but the one query in ten thousand that is handed over then tends to be
-      // one that ends last; query_order = 2 puts any batch of more than one round in order)
       const long long resident = slots;  // queries at work at a time
-      // (and up to 32 rounds: what the order saves is part of one round, what the separate descents cost grows
-      // with the batch — 1 000 000 queries, 145 rounds: 211.7 against 201.9 ms in the caller's order)
       // A handed-over query is not searched again from its entry point: the first pass leaves the entries it
       // accepted, hop by hop, and the literal pass (on the sorted set with ids: it needs no visited bitmap
       // brought up to date) replays its queue operations from them up to where the two may part.  One query per
       // wavefront, link rows of one pass of 64 lanes, and batches of up to two rounds of wavefronts: keeping the
       // trail costs the first pass 2 to 3 %, which only a batch short enough to wait for its last hand-over
-      // gets back (1.18 M x 50, longest first, eight draws of 10 000 queries: 2.75 -> 2.65 ms on average, the
-      // slowest draws 3.06 -> 2.88; 40 000 queries: 6.24 -> 6.39 ms with trails kept).  trails = 2: whatever the batch.
+      // gets back.  trails = 2: whatever the batch.
       bool keep_trails = (QR == 1 || QR == 2) && trails && !a.reverse && a.lean && host.S0 <= 63 &&
                          (trails > 1 || a.nq <= 2 * resident);
       if (keep_trails) {
@@ -639,13 +636,20 @@ class Engine {
         a.trail_next = d_ctl.p + 48;
         a.redo_trail = d_redo_trail.p;
       }
+      {
+        const int n_hist = in_order ? kOrderBuckets : 0;
+        const int n_fill = std::max(std::max(a.nq, n_hist), 128);
+        hipLaunchKernelGGL(prepare_search_kernel, dim3((unsigned)((n_fill + 255) / 256)), dim3(256), 0, stream, d_ctl.p, 128,
+                           d_redo.p, a.nq, in_order ? d_order_hist.p : nullptr, n_hist);
+        HIP_CHECK(hipGetLastError());
+      }
       if (side) {
         SearchArgs b = a;
         b.live = 1;
         b.counter = d_ctl.p + 96;
         b.pool = pool;
         // one or two of these wavefronts per CU: LDS for a candidate queue that never spills costs the first
-        // pass nothing (10 000 queries: 2.98 -> 2.87 ms; the queue of a long search outgrows 2 * ef entries)
+        // pass nothing (the queue of a long search outgrows 2 * ef entries)
         if (NS > 0) b.cand_lds = std::max(a.cand_lds, 1024);
         const LdsPlan lp_side = plan_lds(QR, ix.Dp, NS > 0 ? -1 : a.ef, b.cand_lds, a.lcap, 0, 0, a.lean ? 0 : a.vc_bits, 0, a.lean);
         // (the first pass starts after the batch's descents when its queries are put in order: 0.1 ms per
@@ -664,9 +668,8 @@ class Engine {
         a.entry = d_entry.p;
         a.order = d_order.p;
         a.order_hist = d_order_hist.p;
-        HIP_CHECK(hipMemsetAsync(d_order_hist.p, 0, (size_t)kOrderBuckets * sizeof(int), stream));
         if constexpr (QR == 1 || QR == 2) {
-          // four queries per wavefront, one per group of 16 lanes (40 000 queries: 0.28 -> 0.16 ms)
+          // four queries per wavefront, one per group of 16 lanes
           auto k_entry = entry4_kernel<DT, QR>;
           const int entry_grid = std::max(1, std::min((a.nq + 3) / 4, resident_slots(k_entry, 0)));
           hipLaunchKernelGGL(k_entry, dim3(entry_grid), dim3(64), 0, stream, ix, a);
@@ -693,8 +696,10 @@ class Engine {
       if (side) {
         HIP_CHECK(hipStreamWaitEvent(stream, ev_side1, 0));
       }
-      int ctl[49];
-      HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, sizeof(ctl), hipMemcpyDeviceToHost, stream));
+      HIP_CHECK(hipEventRecord(ev1, stream));  // (recorded again further down if the list has to be answered after all)
+      timed = true;
+      int* ctl = h_ctl;  // pinned: read back without a staging copy
+      HIP_CHECK(hipMemcpyAsync(ctl, d_ctl.p, 49 * sizeof(int), hipMemcpyDeviceToHost, stream));
       HIP_CHECK(hipStreamSynchronize(stream));
       n_literal = last_repeats = ctl[32];
       last_trails = ctl[48];
@@ -719,6 +724,7 @@ class Engine {
       }
     }
     if (n_literal > 0 && !answered) {
+      timed = false;
       SearchArgs b = a;
       b.nq = n_literal;
       int slots = std::max(1, std::min(lit_slots, b.nq));
@@ -740,8 +746,10 @@ class Engine {
       }
       if (!done) throw std::runtime_error("search: candidate queue overflow");
     }
-    HIP_CHECK(hipEventRecord(ev1, stream));
-    HIP_CHECK(hipEventSynchronize(ev1));
+    if (!timed) {
+      HIP_CHECK(hipEventRecord(ev1, stream));
+      HIP_CHECK(hipEventSynchronize(ev1));
+    }
     if (ms) HIP_CHECK(hipEventElapsedTime(ms, ev0, ev1));
   }
   // The search of the entry point that allocates nothing: the sorted-set pass over every query, then the
@@ -897,6 +905,7 @@ class Engine {
     DevBuf<unsigned long long> d_dirty;
     DevBuf<int> d_sel0_cnt, d_selU_cnt, d_inbox0_cnt, d_inboxU_cnt;
     DevBuf<HeapEnt> d_inbox0, d_inboxU;
+    DevBuf<unsigned char> d_selected;  // per link row: the row is an output of the selection rule (kernels.h, BuildArgs)
     d_dists0.reserve((size_t)N * host.S0);
     d_distsU.reserve(up_rows * host.SU);
     d_sel0_ids.reserve((size_t)bmax * host.max_m0);
@@ -911,6 +920,10 @@ class Engine {
     d_inbox0_cnt.reserve((size_t)N);
     d_inboxU.reserve(up_rows * cap_in);
     d_inboxU_cnt.reserve(up_rows);
+    if (newcomer_shortcut) {
+      d_selected.reserve((size_t)N + up_rows);
+      HIP_CHECK(hipMemsetAsync(d_selected.p, 0, (size_t)N + up_rows, stream));
+    }
     HIP_CHECK(hipMemsetAsync(d_inbox0_cnt.p, 0, (size_t)N * 4, stream));
     HIP_CHECK(hipMemsetAsync(d_inboxU_cnt.p, 0, up_rows * 4, stream));
     HIP_CHECK(hipMemsetAsync(d_links0.p, 0xFF, (size_t)N * host.S0 * 4, stream));
@@ -939,6 +952,8 @@ class Engine {
     a.cap_in = cap_in;
     a.dirty = d_dirty.p; a.dirty_cnt = d_ctl.p + 2;
     a.dropped = d_ctl.p + 3;
+    a.selected0 = newcomer_shortcut ? d_selected.p : nullptr;
+    a.selectedU = newcomer_shortcut ? d_selected.p + N : nullptr;
     DevBuf<unsigned long long> d_work;
     if (count_build_work) {
       d_work.reserve(10);
@@ -967,10 +982,9 @@ class Engine {
     // one of all earlier batches: its entry point is the first node that reached the highest
     // level so far.  Batches grow with the graph — a quarter of what is already in, up to 16 384 nodes, so
     // that early nodes, which wire the long-range links, see each other; beyond half a million nodes a
-    // thirty-second of the graph, up to 65 536 — because the nodes of a batch do not see each other, and a
-    // launch of several rounds of wavefronts loses less to its last, partly filled round (1.18 M x 50: 0.224 s
-    // with batches of 16 384 throughout, 0.171 s with 65 536, recall unchanged; 1 M x 960: recall@10 at
-    // ef_search 300 0.9831 / 0.9812, at 50 0.836 / 0.829, which is why the share of new nodes stays small).
+    // thirty-second of the graph, up to 65 536 — because the nodes of a batch do not see each other (recall
+    // falls when the share of new nodes grows), and a launch of several rounds of wavefronts loses less to
+    // its last, partly filled round.
     // build_batch > 0 replaces the two caps by one.
     auto batch_at = [&](int in) {
       if (build_batch > 0) return std::max(1, std::min(build_batch, in / 4));
@@ -1264,6 +1278,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;
   else if (n == "visited_cache") e->impl.visited_cache = (int)value;
   else if (n == "own_links0") e->impl.own_links0 = (int)value;
+  else if (n == "newcomer_shortcut") e->impl.newcomer_shortcut = value != 0.0;
   else if (n == "fast_path") e->impl.fast_path = (int)value;
   else if (n == "lean_literal") e->impl.lean_literal = (int)value;
   else if (n == "trails") e->impl.trails = (int)value;

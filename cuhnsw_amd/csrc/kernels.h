@@ -113,6 +113,12 @@ struct BuildArgs {
   unsigned long long* dirty;  // node | level << 32
   int* dirty_cnt;
   int* dropped;  // reverse links that found no room in an inbox (kept: the cap_in closest newcomers)
+  // Per link row (N level-0 rows, then the upper rows): 1 = the row as it stands is an output of the selection
+  // rule (written by a selection, not appended to since), so that a later re-selection may take the shortcut
+  // for newcomers.  The reference keeps the same fact per node and level as went_through_heuristic
+  // (cpp/include/cuda_build_kernels.cuh:277,322).  Null = no shortcut.
+  unsigned char* selected0;
+  unsigned char* selectedU;
   // optional work counters of a build (null = off), level 0 in [0..4], upper levels in [5..9]:
   //   +0 distance evaluations of the searches and descents (one vector row each)
   //   +1 link rows read (expanded candidates, descent sweeps, rows merged with their inbox)
@@ -836,13 +842,23 @@ __device__ __forceinline__ void load_node_query(QVec<QR>& qv, float4* qlds, cons
 // the first nn_num candidates pass unconditionally, and with save_remains pruned
 // candidates fill the row from the tail.  Candidates sid/skey[0..T) are ascending.
 // Returns the degree; oid/okey[0..degree) is the new row.
+//
+// new_from > 0 is the reference's new_comer shortcut (cuda_build_kernels.cuh:109-110,122-125,137-138) in the
+// form that is exact for any number of newcomers: the candidates with an id below new_from are a row that
+// this very rule produced before (each of them was tested against every pick before it and passed), the
+// others are newcomers.  A newcomer is tested against every pick before it, as always; an old candidate only
+// against the NEWCOMERS picked before it — the old picks before it are a subset of those it has passed
+// already.  Same row as the full rule, at a fraction of its pair tests.  (Only with nn_num = 0 and without
+// save_remains: free picks and tail fill make a row that the rule's own tests do not vouch for.)
 template <int DT, int QR>
 __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32_t* sid, const float* skey, int T, int m,
                                                 int nn_num, int save_remains, uint32_t* oid, float* okey, Scratch& s,
-                                                int lane, unsigned int* work = nullptr) {
+                                                int lane, unsigned int* work = nullptr, uint32_t new_from = 0u) {
   int head = 0;
   int tail = (m < T ? m : T) - 1;
   const int max_head = tail + 1;
+  uint32_t* picked_new = s.nbuf;  // ids of the newcomers picked so far (new_from > 0 only)
+  int n_new = 0;
   // candidates are examined in list order whatever the outcome, so the next candidate's
   // vector can be fetched while the current one is being tested (register copy; for long
   // rows the LDS copy is filled when the candidate comes up)
@@ -855,22 +871,30 @@ __device__ __forceinline__ int select_neighbors(const DevIndex& ix, const uint32
     bool skip = false;
     QVec<QR> cv = cv_next;
     if (QR > 0 && j + 1 < T) load_node_query<QR>(cv_next, s.qlds, ix, sid[j + 1], lane);
-    if (head >= nn_num && head > 0) {
+    const bool newcomer = c >= new_from;  // (new_from = 0: every candidate gets the full test)
+    const uint32_t* against = newcomer ? oid : picked_new;
+    const int n_against = newcomer ? head : n_new;
+    if (head >= nn_num && n_against > 0) {
       if (QR == 0) load_node_query<QR>(cv, s.qlds, ix, c, lane);
       if (work && lane == 0) {  // (LDS: +2 pair tests, +3 candidate rows of this level's counters)
-        work[2] += (unsigned int)head;
+        work[2] += (unsigned int)n_against;
         work[3] += 1u;
       }
-      dist_list<DT, QR, false>(ix, cv, s.qlds, oid, head, s.dbuf, lane);
+      dist_list<DT, QR, false>(ix, cv, s.qlds, against, n_against, s.dbuf, lane);
       wave_sync();
       bool mine = false;
-      for (int t = lane; t < head; t += 64) mine = mine || (dq > s.dbuf[t]);
+      for (int t = lane; t < n_against; t += 64) mine = mine || (dq > s.dbuf[t]);
       skip = __ballot(mine) != 0ull;
       wave_sync();
     }
     if (!skip) {
-      if (lane == 0) { oid[head] = c; okey[head] = dq; }
+      if (lane == 0) {
+        oid[head] = c;
+        okey[head] = dq;
+        if (new_from > 0u && newcomer) picked_new[n_new] = c;
+      }
       head++;
+      if (new_from > 0u && newcomer) n_new++;
     } else if (tail >= head) {
       if (lane == 0) { oid[tail] = c; okey[tail] = dq; }
       tail--;
@@ -1059,6 +1083,12 @@ __global__ void __launch_bounds__(256) apply_kernel(DevIndex ix, BuildArgs a) {
     const float key = sel_keys[j];
     link_row_mut(ix, x, level)[j] = y;
     dist_row_mut(ix, x, level)[j] = key;
+    if (j == 0 && a.selected0) {
+      // (with free picks or the tail fill the row holds entries the rule's tests do not vouch for)
+      const unsigned char pure = (level == 0 ? a.nn_num0 : a.nn_numU) == 0 && !a.save_remains;
+      if (level == 0) a.selected0[x] = pure;
+      else a.selectedU[(size_t)(ix.upper_off[x] + level - 1)] = pure;
+    }
     if (j < deg) {
       int* cnt;
       HeapEnt* box;
@@ -1243,6 +1273,8 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
     wave_sync();
     const int n_new = T - n0;
     if (n_new > 0) {
+      unsigned char* selected = !a.selected0 ? nullptr
+                                : (level == 0 ? a.selected0 + y : a.selectedU + (size_t)(ix.upper_off[y] + level - 1));
       if (T <= m_cap) {
         // room for all: append the newcomers, ordered by (key, id)
         rank_sort(cbuf + n0, nullptr, n_new, sid, skey, lane);
@@ -1251,16 +1283,23 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
           row[n0 + t] = sid[t];
           drow[n0 + t] = skey[t];
         }
+        if (selected && lane == 0) *selected = 0;  // no longer what the selection rule alone would leave
       } else {
         rank_sort(cbuf, nullptr, T, sid, skey, lane);
         wave_sync();
-        const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, m_cap, level == 0 ? a.nn_num0 : a.nn_numU,
-                                                 a.save_remains, oid, okey, s, lane,
-                                                 a.counters ? work + (level == 0 ? 0 : 5) : nullptr);
+        // A row that is an output of the rule is re-selected with the shortcut for newcomers: the nodes of this
+        // batch (ids from a.begin on; everything the row held before has a smaller id).
+        const int nn_num = level == 0 ? a.nn_num0 : a.nn_numU;
+        const bool pure = nn_num == 0 && !a.save_remains;
+        const bool shortcut = pure && selected && uni((int)*selected) != 0;
+        const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, m_cap, nn_num, a.save_remains, oid, okey, s, lane,
+                                                 a.counters ? work + (level == 0 ? 0 : 5) : nullptr,
+                                                 shortcut ? (uint32_t)a.begin : 0u);
         for (int j = lane; j < m_cap; j += 64) {
           row[j] = j < deg ? oid[j] : kEmpty;
           drow[j] = j < deg ? okey[j] : 0.f;
         }
+        if (selected && lane == 0) *selected = pure ? 1 : 0;
       }
     }
     if (lane == 0) *cnt = 0;

@@ -215,6 +215,11 @@ int cuhnsw_trails_available(cuhnsw_engine* e);
  *   "trail_cap"     accepted entries a trail holds (default 2048; a search that accepts more leaves none)
  *   "trail_spares"  handed-over queries per batch that can come with a trail (default 1024: each keeps the
  *                   buffer it was written to until the batch is over; the ones after that come without)
+ *   "newcomer_shortcut" 1 (default) = a link row that the selection rule itself produced is re-selected, when
+ *                   an insertion batch brings it newcomers, with the reference's new_comer shortcut
+ *                   (cpp/include/cuda_build_kernels.cuh:109-138): its old entries are tested only against the
+ *                   newcomers picked before them.  Same graph byte for byte, fewer pair tests; 0 = the full
+ *                   rule on every re-selection.  Applies with heuristic_coef = 0 and save_remains = false.
  *   "own_links0"    most links a newly inserted node selects for itself on level 0
  *                   (0 = max_m0, as cpp/src/cuhnsw_build.cu:110 does; hnswlib's addPoint uses
  *                   max_m there and max_m0 only as the room for reverse links)

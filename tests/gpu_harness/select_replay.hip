@@ -18,6 +18,7 @@ struct SelectCases {
   const int* m;               // per case: row capacity
   const int* nn_num;          // per case: picks that pass untested
   const int* save_remains;    // per case
+  const uint32_t* new_from;   // per case: candidates with ids from here on are newcomers to a row the rule produced (0 = none)
   uint32_t* out_ids;          // n_cases x cap
   float* out_keys;
   int* out_deg;
@@ -44,7 +45,8 @@ __global__ void __launch_bounds__(64) select_kernel(DevIndex ix, SelectCases c) 
       skey[t] = c.cand_keys[beg + t];
     }
     wave_sync();
-    const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, c.m[i], c.nn_num[i], c.save_remains[i], oid, okey, s, lane);
+    const int deg = select_neighbors<DT, QR>(ix, sid, skey, T, c.m[i], c.nn_num[i], c.save_remains[i], oid, okey, s, lane,
+                                             nullptr, c.new_from[i]);
     wave_sync();
     for (int j = lane; j < c.cap; j += 64) {
       c.out_ids[(size_t)i * c.cap + j] = j < deg ? oid[j] : kEmpty;
@@ -84,7 +86,8 @@ static T* upload(const std::vector<T>& v) {
 // vectors: N x D fp32 (already rounded to fp16 values when half != 0).  Returns 0 on success.
 extern "C" int select_replay(const float* vectors, int N, int D, int dist_type, int half, int n_cases, const unsigned* cand_ids,
                              const float* cand_keys, const int* cand_off, const int* m, const int* nn_num,
-                             const int* save_remains, int cap, unsigned* out_ids, float* out_keys, int* out_deg) {
+                             const int* save_remains, const unsigned* new_from, int cap, unsigned* out_ids, float* out_keys,
+                             int* out_deg) {
   const int Dp = padded_dims(D);
   DevIndex ix{};
   void* d_vec = nullptr;
@@ -118,6 +121,7 @@ extern "C" int select_replay(const float* vectors, int N, int D, int dist_type, 
   c.m = upload(std::vector<int>(m, m + n_cases));
   c.nn_num = upload(std::vector<int>(nn_num, nn_num + n_cases));
   c.save_remains = upload(std::vector<int>(save_remains, save_remains + n_cases));
+  c.new_from = upload(std::vector<uint32_t>(new_from, new_from + n_cases));
   c.out_ids = upload(std::vector<uint32_t>((size_t)n_cases * cap, 0u));
   c.out_keys = upload(std::vector<float>((size_t)n_cases * cap, 0.f));
   c.out_deg = upload(std::vector<int>(n_cases, 0));
@@ -134,6 +138,6 @@ extern "C" int select_replay(const float* vectors, int N, int D, int dist_type, 
   (void)hipFree(d_vec);
   (void)hipFree(const_cast<uint32_t*>(c.cand_ids)); (void)hipFree(const_cast<float*>(c.cand_keys));
   (void)hipFree(const_cast<int*>(c.cand_off)); (void)hipFree(const_cast<int*>(c.m)); (void)hipFree(const_cast<int*>(c.nn_num));
-  (void)hipFree(const_cast<int*>(c.save_remains)); (void)hipFree(c.out_ids); (void)hipFree(c.out_keys); (void)hipFree(c.out_deg);
+  (void)hipFree(const_cast<int*>(c.save_remains)); (void)hipFree(const_cast<uint32_t*>(c.new_from)); (void)hipFree(c.out_ids); (void)hipFree(c.out_keys); (void)hipFree(c.out_deg);
   return rc;
 }

@@ -160,6 +160,35 @@ def test_build_is_deterministic(tmp_path):
   assert files[0] == files[1]
 
 
+def test_newcomer_shortcut_builds_the_same_graph_with_fewer_pair_tests(tmp_path):
+  """A link row that the selection rule produced is re-selected, when a batch brings it newcomers, with the
+  reference's new_comer shortcut (old entries are tested against the picked newcomers only): the same file byte for
+  byte as with the full rule on every re-selection, and fewer pair tests on the device's own counters — on
+  clustered and on tie-heavy integer data."""
+  from cuhnsw_amd import capi
+  for kind, n, d, dist, max_m in (("gauss", 40000, 50, "dot", 12), ("int", 15000, 128, "l2", 16)):
+    x = _data(kind, n, d, 61)
+    levels = _levels(n, 1.0 / np.log(max_m), 62)
+    path, _ = write_options(tmp_path, dist_type=dist, max_m=max_m, max_m0=2 * max_m, ef_construction=100, heuristic_coef=0.0)
+    files, tests = {}, {}
+    for shortcut in (1, 0):
+      e = capi.Engine()
+      assert e.init(path) == 0
+      e.set_tunable("newcomer_shortcut", shortcut)
+      e.set_tunable("build_counters", 1)
+      e.set_data(x)
+      e.set_random_levels(levels)
+      e.build_graph()
+      c = e.build_counters()
+      tests[shortcut] = c["level0"][2] + c["upper"][2]
+      p = str(tmp_path / ("nc_%s_%d.idx" % (kind, shortcut)))
+      e.save_index(p)
+      files[shortcut] = open(p, "rb").read()
+    print("pair tests", kind, "with the shortcut", tests[1], "without", tests[0], flush=True)
+    assert files[1] == files[0]
+    assert tests[1] < tests[0]
+
+
 def test_hand_out_order_and_batch_cap_tunables(oracle, tmp_path):
   """Which node of a batch a wavefront takes next (upper-level nodes first, or by id) cannot change the graph: the
   batch reads the graph of the earlier batches only.  The batch cap can: a single cap of 2 000 nodes is another
