@@ -128,6 +128,10 @@ __device__ __forceinline__ float uni(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
 }
 __device__ __forceinline__ int uni(int x) { return __builtin_amdgcn_readfirstlane(x); }
+// how many lanes below this one have their bit set in a wavefront-uniform mask (v_mbcnt: no lane masks in registers)
+__device__ __forceinline__ int lanes_below(unsigned long long mask) {
+  return (int)__builtin_amdgcn_mbcnt_hi((unsigned int)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned int)mask, 0u));
+}
 __device__ __forceinline__ float wave_min(float x) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) x = fminf(x, __shfl_xor(x, m, 64));
@@ -373,7 +377,7 @@ __device__ __forceinline__ int visit_row(const uint32_t* row, int S, Scratch& s,
       if (s.vcache != nullptr) s.vcache[slot] = tag;
     }
     unsigned long long mask = __ballot(newly);
-    int pos = n + __popcll(mask & ((1ull << lane) - 1ull));
+    int pos = n + lanes_below(mask);
     if (newly) {
       s.nbuf[pos] = id;
       int u = st.undo_cnt + pos;
@@ -410,7 +414,7 @@ __device__ __forceinline__ VisitPending visit_issue(const uint32_t* row, int S, 
     v.ask = s.vcache[slot] != tag;
   }
   const unsigned long long mask = __ballot(v.ask);
-  v.pos = __popcll(mask & ((1ull << lane) - 1ull));
+  v.pos = lanes_below(mask);
   v.n_ask = __popcll(mask);
   v.bit = 1u << (v.id & 31);
   v.old = 0u;
@@ -426,7 +430,7 @@ __device__ __forceinline__ int visit_commit(const VisitPending& v, Scratch& s, S
   const unsigned long long mask = __ballot(newly);
   if (v.ask && !newly) s.nbuf[v.pos] = kEmpty;
   if (newly) {
-    const int u = st.undo_cnt + __popcll(mask & ((1ull << lane) - 1ull));
+    const int u = st.undo_cnt + lanes_below(mask);
     if (u < s.undo_cap) s.undo[u] = v.id;
   }
   const int n_new = __popcll(mask);
@@ -441,7 +445,7 @@ __device__ __forceinline__ int load_row(const uint32_t* row, int S, Scratch& s, 
     uint32_t id = (base + lane < S) ? row[base + lane] : kEmpty;
     bool valid = id != kEmpty;
     unsigned long long mask = __ballot(valid);
-    int pos = n + __popcll(mask & ((1ull << lane) - 1ull));
+    int pos = n + lanes_below(mask);
     if (valid) s.nbuf[pos] = id;
     n += __popcll(mask);
   }
@@ -798,6 +802,56 @@ __device__ __forceinline__ bool frontier_tie_within(const Frontier<NS>& f, int e
   }
   return __ballot(hit) != 0ull;
 }
+// The waiting (not yet expanded) entries whose key coincides with a neighbour's: while the tie-free loop runs on a
+// set that holds equal keys, these are the entries it must not expand or push out by itself.
+struct TieWatch {
+  int id0 = -1, id1 = -1, id2 = -1, id3 = -1;  // (-1: unused; no taken candidate compares equal)
+  float hi = -INFINITY;                        // their largest key
+};
+// Fills w; false when there are more than four such entries.
+template <int NS>
+__device__ __forceinline__ bool frontier_watch_list(const Frontier<NS>& f, TieWatch& w) {
+  constexpr int N = NS > 0 ? NS : 1;
+  const float prev_last = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, f.k[N - 1]), 0x138, 0xF, 0xF, false));  // wave_shr:1
+  const float next_first = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, f.k[0]), 0x130, 0xF, 0xF, false));  // wave_shl:1
+  unsigned long long m[N];
+  int total = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    const float below = j > 0 ? f.k[j > 0 ? j - 1 : 0] : prev_last;
+    const float above = j + 1 < N ? f.k[j + 1 < N ? j + 1 : 0] : next_first;
+    m[j] = __ballot((f.v[j] & kExpanded) == 0u && (f.k[j] == below || f.k[j] == above));
+    total += __popcll(m[j]);
+  }
+  w = TieWatch();
+  if (total > 4) return false;
+  int cnt = 0;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    while (m[j] != 0ull) {
+      const int L = __builtin_ctzll(m[j]);
+      m[j] &= m[j] - 1ull;
+      const int id = __builtin_amdgcn_readlane((int)f.v[j], L);
+      const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f.k[j]), L));
+      if (cnt == 0) w.id0 = id;
+      else if (cnt == 1) w.id1 = id;
+      else if (cnt == 2) w.id2 = id;
+      else w.id3 = id;
+      w.hi = uni(fmaxf(w.hi, key));
+      cnt += 1;
+    }
+  }
+  return true;
+}
+// takes the expanded mark off an entry again
+template <int NS>
+__device__ __forceinline__ void frontier_untake(Frontier<NS>& f, uint32_t id) {
+  constexpr int N = NS > 0 ? NS : 1;
+#pragma unroll
+  for (int j = 0; j < N; ++j) f.v[j] = f.v[j] == (id | kExpanded) ? id : f.v[j];
+}
 // writes the sorted entries [0, count) to out_id / out_key (LDS)
 template <int NS>
 __device__ __forceinline__ void frontier_dump(const Frontier<NS>& f, int ef, int count, uint32_t* out_id, float* out_key,
@@ -851,7 +905,7 @@ __device__ __forceinline__ int visit_lossy(const uint32_t* row, int S, Scratch& 
     const unsigned long long mask = __ballot(ask);
     if (ask) {
       sets[slot] = filter_push(w, tag);
-      s.nbuf[n + __popcll(mask & ((1ull << lane) - 1ull))] = id;
+      s.nbuf[n + lanes_below(mask)] = id;
     }
     n += __popcll(mask);
   }
@@ -888,6 +942,10 @@ struct Trail {
   bool on = false;   // still recording
   bool own = false;  // inside a stretch the literal pass makes itself
 };
+// (The wave barriers after the one-lane and some-lanes stores below emit nothing; they keep the end of such a
+// branch a block of its own.  Merged into the join of the surrounding wavefront-uniform branches, it makes the
+// compiler take every value that differs between those for lane-dependent -- the trail's state then sits in
+// vector registers, of which the pass has none to spare.)
 __device__ __forceinline__ void trail_mark(Trail& tr, uint32_t kind, int hop, int lane) {
   if (tr.on) {
     if (tr.n + 1 > tr.cap) {
@@ -895,6 +953,7 @@ __device__ __forceinline__ void trail_mark(Trail& tr, uint32_t kind, int hop, in
       tr.n = -1;
     } else {
       if (lane == 0) tr.rec[tr.n] = make_uint4(kind, 0u, 0u, (uint32_t)hop);
+      __builtin_amdgcn_wave_barrier();
       tr.n += 1;
       tr.own = kind == kTrailOwn;
     }
@@ -908,10 +967,10 @@ __device__ __forceinline__ void trail_hop(Trail& tr, unsigned long long accepted
       tr.on = false;
       tr.n = -1;
     } else {
-      if ((accepted >> lane) & 1ull) {
-        const int at = tr.n + __popcll(accepted & ((1ull << lane) - 1ull));
-        tr.rec[at] = make_uint4((uint32_t)cid, my_id, __float_as_uint(my_key), (uint32_t)hop);
+      if (__builtin_amdgcn_inverse_ballot_w64(accepted)) {  // (the lanes whose bit is set)
+        tr.rec[tr.n + lanes_below(accepted)] = make_uint4((uint32_t)cid, my_id, __float_as_uint(my_key), (uint32_t)hop);
       }
+      __builtin_amdgcn_wave_barrier();
       tr.n += cnt;
     }
   }
@@ -934,11 +993,15 @@ __device__ __forceinline__ void trail_stop(Trail& tr, int hops, int n_dist) {
 // nothing for them).  Returns 0: no waiting entry is left, the search is over; 1: an
 // offer met an equal key of another node (resume_at = which offer of the list in s.nbuf / s.dbuf); 2 (FULL = false
 // only): the set is full now, the other phase goes on.  n = ids waiting in s.nbuf on entry.
-template <int DT, int QR, int NS, bool FULL, bool TRAILS>
+template <int DT, int QR, int NS, bool FULL, bool TRAILS, bool WATCH>
 __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, int S, Scratch& s,
                                               SearchState& st, Frontier<NS>& fr, int& n, int& hop_cid, int& resume_at,
-                                              unsigned long long& accepted, Trail& tr, int lane) {
+                                              unsigned long long& accepted, Trail& tr, const TieWatch& watch, int lane) {
   constexpr int N = NS > 0 ? NS : 1;
+  // (said to be wavefront-uniform, so that they sit in scalar registers through the loop)
+  const int w0 = WATCH ? uni(watch.id0) : -1, w1 = WATCH ? uni(watch.id1) : -1;
+  const int w2 = WATCH ? uni(watch.id2) : -1, w3 = WATCH ? uni(watch.id3) : -1;
+  const float w_hi = WATCH ? uni(watch.hi) : -INFINITY;
   while (true) {
     if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
     st.n_dist += n;
@@ -959,6 +1022,9 @@ __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>
         bool eq = false;
 #pragma unroll
         for (int t = 0; t < N; ++t) eq = eq || fr.k[t] == key;
+        // (WATCH: an eviction that would reach a watched entry, or its equal, is the general loop's as well)
+        // (while the set is not full its last key is the padding's +inf)
+        if (WATCH) eq = eq || (lane == 63 && fr.k[N - 1] <= w_hi);
         if (__ballot(eq) == 0ull) {
           frontier_insert_distinct<NS>(fr, key, id);
           if (TRAILS) accepted |= 1ull << j;
@@ -974,7 +1040,7 @@ __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>
 #pragma unroll
           for (int t = 0; t < N; ++t) same = same || (fr.k[t] == key && (fr.v[t] & ~kExpanded) == id);
           if (__ballot(same) == 0ull) {
-            resume_at = j;  // an equal key of another node: the rules for equal keys apply from this offer on
+            resume_at = j;  // an equal key of another node (WATCH: or a watched eviction): the rules for equal keys apply from this offer on
             todo = 0ull;
           }
           // (else: a node met again after the visited filter forgot it; it is in the set already)
@@ -986,6 +1052,11 @@ __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>
     accepted = 0ull;
     const int cid = frontier_take<NS>(fr, lane, false);
     if (cid < 0) return 0;
+    if (WATCH && (cid == w0 || cid == w1 || cid == w2 || cid == w3)) {
+      frontier_untake<NS>(fr, (uint32_t)cid);  // a watched entry's turn: the general loop takes it, with its bookkeeping
+      n = 0;
+      return 3;
+    }
     hop_cid = cid;
     st.n_hops += 1;
     wave_sync();
@@ -1055,14 +1126,33 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   // instructions per accepted candidate — and only then moves on to the general loop below, at the very offer
   // that met the equal key (resume_at).
   int resume_at = -1;
-  if (exact && S <= 64) {
-    int how = st.n_acc >= ef ? 2 : tie_free_phase<DT, QR, NS, false, TRAILS>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, lane);
-    if (how == 2) how = tie_free_phase<DT, QR, NS, true, TRAILS>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, lane);
+  bool calm = exact && S <= 64;  // no equal keys are at work: the tie-free loop may run
+  TieWatch watch;
+  while (true) {
+  if (calm) {
+    int how = st.n_acc >= ef ? 2 : 0;
+    if (!have_tie) {
+      if (how == 0) how = tie_free_phase<DT, QR, NS, false, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+      if (how == 2) how = tie_free_phase<DT, QR, NS, true, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+    } else {
+      // (after equal keys have met, the tie-free loop takes over again only once the set is full: how == 2)
+      how = tie_free_phase<DT, QR, NS, true, TRAILS, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+    }
     st.top_size = st.n_acc < ef ? st.n_acc : ef;
     if (how == 0) {
       trail_stop(tr, st.n_hops, st.n_dist);
-      return 0;
+      return have_tie ? 2 : 0;
     }
+    calm = false;
+    // (what these were when the tie-free loop took over; said again so that none of them has to live through it)
+    ghosts = 0;
+    ghost = kEmpty;
+    twin_phase = false;
+    in_group = false;
+    group_key = 0.f;
+    group_edge = INFINITY;
+    ek_min = INFINITY;
+    gave_up = false;
   }
   while (true) {
     if (resume_at < 0) {
@@ -1187,6 +1277,21 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
     wave_sync();
     n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
     wave_sync();
+    // Equal keys that sit in the set do no harm while none of them that still waits is expanded or pushed out
+    // (unless the whole set is the answer): no group can form, and which of two expanded twins an eviction
+    // pushes out changes neither the keys of the set nor hnswlib's candidates.  With no group under way and
+    // no eviction out of equal largest keys on record whose key is still within the bound (once the bound is
+    // below it, the entry such an eviction pushed out is as dead for hnswlib as any other), the tie-free loop
+    // takes over again from this hop's offers, with the waiting entries that have an equal (at most four) on
+    // its watch list; it comes back at the next offer that meets an equal key, when a watched entry's turn
+    // comes, or when an eviction reaches one.
+    if (exact && S <= 64 && !whole_set && st.n_acc >= ef && !in_group && !twin_phase && (ghosts == 0 || st.lower < ek_min) &&
+        frontier_watch_list<NS>(fr, watch)) {
+      calm = true;
+      break;
+    }
+  }
+  if (!calm) break;
   }
   return gave_up ? 1 : (have_tie ? 2 : 0);
 }
@@ -1441,7 +1546,7 @@ __device__ __forceinline__ int collect_le(const HeapEnt* log, int n, float bound
     if (i < n) e = log[i];
     const bool keep = i < n && e.key <= bound;
     const unsigned long long mask = __ballot(keep);
-    const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+    const int pos = cnt + lanes_below(mask);
     if (keep && pos < cap) out[pos] = e;
     cnt += __popcll(mask);
   }
@@ -1460,7 +1565,7 @@ __device__ __forceinline__ int collect_best(const HeapEnt* log, int n, float bou
       if (i < n) e = log[i];
       const bool keep = i < n && (pass == 0 ? e.key < bound : e.key == bound);
       const unsigned long long mask = __ballot(keep);
-      const int pos = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+      const int pos = cnt + lanes_below(mask);
       if (keep && pos < want) out[pos] = e;
       cnt += __popcll(mask);
     }

@@ -468,6 +468,9 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2) ? (NS <= 5 ? 7 : (NS 
         __hip_atomic_store(&a.redo[slot], qi, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         if (with_trail) spare = atomicAdd(a.trail_next, 1);
       }
+      // (the lanes meet again HERE: threaded through to the loop's end, lane 0's way out of the branch above
+      // would make everything the next lines set look lane-dependent to the compiler)
+      __builtin_amdgcn_wave_barrier();
       if (with_trail) {
         // that buffer belongs to the literal pass now
         spare = __builtin_amdgcn_readfirstlane(spare);
@@ -1249,7 +1252,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
       float key = (base + lane < S) ? drow[base + lane] : 0.f;
       bool valid = id != kEmpty;
       unsigned long long mask = __ballot(valid);
-      int pos = n0 + __popcll(mask & ((1ull << lane) - 1ull));
+      int pos = n0 + lanes_below(mask);
       if (valid) { cbuf[pos].key = key; cbuf[pos].id = id; }
       n0 += __popcll(mask);
     }
@@ -1266,7 +1269,7 @@ __global__ void __launch_bounds__(64) reverse_kernel(DevIndex ix, BuildArgs a) {
         for (int t = 0; t < n0; ++t) keep = keep && (cbuf[t].id != e.id);
       }
       unsigned long long mask = __ballot(keep);
-      int pos = T + __popcll(mask & ((1ull << lane) - 1ull));
+      int pos = T + lanes_below(mask);
       if (keep) cbuf[pos] = e;
       T += __popcll(mask);
     }

@@ -5,8 +5,8 @@ SIMD; a register spilled INSIDE its hop loop (a scratch reload per hop, and the 
 the pass 7 to 12 %, and whether the register allocator puts one there is decided by small changes anywhere
 in the kernel.  This module compiles the kernels that matter on their own (a few seconds each), reads
 hipcc's resource-usage remarks (registers, spills, scratch bytes, wavefronts per SIMD) and counts the
-scratch-memory instructions that sit inside the loops holding the sorted-set insert (`v_med3_f32`), from
-the control-flow graph of the emitted ISA.
+scratch-memory instructions that sit inside the hop loops (the innermost loops holding both the sorted-set
+insert, `v_med3_f32`, and a fetch from global memory), from the control-flow graph of the emitted ISA.
 
   python -m cuhnsw_amd.kernel_report            # prints the table
 
@@ -86,8 +86,8 @@ def _blocks(body):
 
 
 def loop_scratch_accesses(isa_text, mangled):
-  """Scratch-memory instructions inside the loops (strongly connected components of the control-flow graph) that
-  contain the sorted-set insert, and in the whole kernel: (in_loops, total)."""
+  """Scratch-memory instructions inside the hop loops (found as strongly connected components of the control-flow
+  graph, nested), and in the whole kernel: (in_loops, total)."""
   start = isa_text.index("\n" + mangled + ":")
   body = isa_text[start:isa_text.index(".Lfunc_end", start)]
   blocks = _blocks(body)
@@ -152,45 +152,29 @@ def loop_scratch_accesses(isa_text, mangled):
           low[parent] = min(low[parent], low[v])
     return comps
 
-  depth = [0] * len(blocks)
-  def nest(nodes, edges, level):
+  # Hop loops: the innermost loops that hold both the sorted-set insert (v_med3_f32) and a fetch from global
+  # memory (the link row, the vectors).  The loop over the wavefront's queries and any loop that merely
+  # alternates between two hop loops contain such a loop and are not counted themselves; the loop over a hop's
+  # offers holds the insert but fetches nothing.
+  has_insert = [any(t.startswith("v_med3_f32") for t in ins) for _, ins in blocks]
+  has_fetch = [any(t.startswith("global_load") for t in ins) for _, ins in blocks]
+  hot_blocks = set()
+  def nest(nodes, edges):
+    """Marks the hop loops inside `nodes`; returns whether there was one."""
+    found = False
     for comp in components(nodes, edges):
       if len(comp) == 1 and next(iter(comp)) not in edges[next(iter(comp))]:
         continue
-      for v in comp:
-        depth[v] = max(depth[v], level)
+      if not (any(has_insert[v] for v in comp) and any(has_fetch[v] for v in comp)):
+        continue
       # headers: nodes of the component entered from outside it (or the first one)
       heads = {v for v in comp for u in range(len(blocks)) if u not in comp and v in succ[u]} or {min(comp)}
       inner = {v: [w for w in edges[v] if w not in heads] for v in comp}
-      nest(comp, inner, level + 1)
-  nest(set(range(len(blocks))), {i: succ[i] for i in range(len(blocks))}, 1)
-  has_insert = [any(t.startswith("v_med3_f32") for t in ins) for _, ins in blocks]
-  # a block belongs to a hop loop if it sits at depth >= 2 in a depth-2 loop that holds an insert: mark by
-  # flooding from the insert blocks inside the depth >= 2 subgraph
-  hot = set(i for i in range(len(blocks)) if has_insert[i] and depth[i] >= 2)
-  deep = {i for i in range(len(blocks)) if depth[i] >= 2}
-  pred = {i: [] for i in deep}
-  for u in deep:
-    for w in succ[u]:
-      if w in deep:
-        pred[w].append(u)
-  frontier = list(hot)
-  fwd = set(hot)
-  while frontier:
-    v = frontier.pop()
-    for w in succ[v]:
-      if w in deep and w not in fwd:
-        fwd.add(w)
-        frontier.append(w)
-  frontier = list(hot)
-  bwd = set(hot)
-  while frontier:
-    v = frontier.pop()
-    for w in pred[v]:
-      if w not in bwd:
-        bwd.add(w)
-        frontier.append(w)
-  hot_blocks = fwd & bwd   # on a cycle through an insert block that stays inside the deeper loops
+      if not nest(comp, inner):
+        hot_blocks.update(comp)
+      found = True
+    return found
+  nest(set(range(len(blocks))), {i: succ[i] for i in range(len(blocks))})
   in_loops = total = 0
   for i, (_, ins) in enumerate(blocks):
     k = sum(1 for t in ins if t.startswith("scratch_"))

@@ -35,6 +35,8 @@ def sorted_set_search(keys_of, rows, ep, k, ef, trail=None):
   S = [[keys_of(ep), ep, False]]          # sorted by key, equal keys in order of arrival
   seen = {ep}
   have_tie = in_group = False
+  calm = True                             # no equal keys at work: the tie-free loop runs (none of the bookkeeping below)
+  watch = []                              # ...keeping off the waiting entries that have an equal in the set (at most four)
   group_key = 0.0
   group_edge = INF                        # smallest key rejected or evicted while the group is expanded
   ek_min = INF
@@ -51,10 +53,13 @@ def sorted_set_search(keys_of, rows, ep, k, ef, trail=None):
         if in_group:
           group_edge = min(group_edge, key)
         continue
-      twins = have_tie and full and S[-1][0] == S[-2][0]   # eviction with equal largest keys to choose from
-      last = list(S[-1])
       if any(e[0] == key for e in S):
         have_tie = True
+        calm = False                          # the rules for equal keys apply from this very offer on
+      if calm and full and watch and S[-1][0] <= max(w[0] for w in watch):
+        calm = False                          # an eviction that reaches a watched entry or its equal
+      twins = not calm and full and S[-1][0] == S[-2][0]   # eviction with equal largest keys to choose from
+      last = list(S[-1])
       pos = len(S)
       while pos > 0 and S[pos - 1][0] > key:
         pos -= 1
@@ -111,7 +116,9 @@ def sorted_set_search(keys_of, rows, ep, k, ef, trail=None):
               offers.append((keys_of(nb), nb))
           continue
       break
-    if have_tie:
+    if calm and pick >= 0 and any(w is S[pick] for w in watch):
+      calm = False                            # a watched entry's turn
+    if have_tie and not calm:
       if d >= ek_min:
         # the twin the set kept (its last entry: the key is the bound)
         others = any((not e[2]) and e[0] == d for i, e in enumerate(S) if i != pick)
@@ -137,6 +144,18 @@ def sorted_set_search(keys_of, rows, ep, k, ef, trail=None):
       if nb not in seen:
         seen.add(nb)
         offers.append((keys_of(nb), nb))
+    # equal keys do no harm while none of them that still waits is expanded or pushed out (unless the whole set
+    # is the answer): once the set is full the tie-free loop takes over again until the next offer meets an equal
+    # key, a watched entry's turn comes or an eviction reaches one
+    if not calm and k < ef and len(S) >= ef and not in_group and not twin_phase and (ghosts == 0 or S[-1][0] < ek_min):
+      watch = [e for i, e in enumerate(S)
+               if (not e[2]) and ((i > 0 and S[i - 1][0] == e[0]) or (i + 1 < len(S) and S[i + 1][0] == e[0]))]
+      if len(watch) <= 4:
+        calm = True
+        sorted_set_search.calmed_down_past_a_ghost += ghosts != 0
+        ghosts, ghost, ek_min = 0, None, INF  # (an eviction out of equal largest keys on record is beyond the bound: dead)
+        sorted_set_search.calmed_down += 1
+        sorted_set_search.calmed_down_watching += bool(watch)
   T = min(k, len(S))
   if have_tie and T < len(S) and S[T - 1][0] == S[T][0]:
     return None                               # equal keys across the cut: the result heap's choice (the trail is complete)
@@ -146,6 +165,9 @@ def sorted_set_search(keys_of, rows, ep, k, ef, trail=None):
 
 
 sorted_set_search.answered_after_twins = 0    # (statistics for the test below: the twin rule has to be exercised)
+sorted_set_search.calmed_down = 0             # (and so has the return to the tie-free loop,
+sorted_set_search.calmed_down_watching = 0    # with and without entries to watch,
+sorted_set_search.calmed_down_past_a_ghost = 0  # and after an eviction out of equal largest keys)
 
 
 def _push_heap(h, value):
@@ -339,3 +361,5 @@ def test_rules_never_let_an_order_dependent_case_through(oracle, seed):
   # by following the twins of an eviction through
   assert answered > 1000 and given_up > 100 and answered_with_ties > 300, (answered, given_up, answered_with_ties)
   assert sorted_set_search.answered_after_twins > 0
+  assert sorted_set_search.calmed_down > 100 and sorted_set_search.calmed_down_watching > 100
+  assert sorted_set_search.calmed_down_past_a_ghost > 20
