@@ -135,7 +135,7 @@ __device__ __forceinline__ int lanes_below(unsigned long long mask) {
 __device__ __forceinline__ float wave_min(float x) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) x = fminf(x, __shfl_xor(x, m, 64));
-  return x;
+  return uni(x);  // (the same in every lane: said so, or all that depends on it counts as lane-dependent)
 }
 
 template <int DT>
@@ -244,6 +244,8 @@ __device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, uin
     const int idx = r + 4 * u + g;
     if (sub == 0 && idx < n) out[idx] = key;
   }
+  // (the lanes meet again here, not at the caller's loop end: see trail_mark)
+  __builtin_amdgcn_wave_barrier();
 }
 
 // long rows: 16 lanes still own one row (the summation order is tied to 16 lanes), so a lane
@@ -279,6 +281,7 @@ __device__ __forceinline__ void dist_long(const void* rows, int rowlen, int used
     }
     const float key = finish16<DT, RAW>(ax, ay, az, aw);
     if (sub == 0 && idx < n) out[idx] = key;
+    __builtin_amdgcn_wave_barrier();  // (the lanes meet again here, not at the loop's end: see trail_mark)
   }
 }
 
@@ -993,7 +996,7 @@ __device__ __forceinline__ void trail_stop(Trail& tr, int hops, int n_dist) {
 // nothing for them).  Returns 0: no waiting entry is left, the search is over; 1: an
 // offer met an equal key of another node (resume_at = which offer of the list in s.nbuf / s.dbuf); 2 (FULL = false
 // only): the set is full now, the other phase goes on.  n = ids waiting in s.nbuf on entry.
-template <int DT, int QR, int NS, bool FULL, bool TRAILS, bool WATCH>
+template <int DT, int QR, int NS, bool FULL, bool TRAILS, bool WATCH, bool BUILD = false>
 __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, int S, Scratch& s,
                                               SearchState& st, Frontier<NS>& fr, int& n, int& hop_cid, int& resume_at,
                                               unsigned long long& accepted, Trail& tr, const TieWatch& watch, int lane) {
@@ -1040,8 +1043,20 @@ __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>
 #pragma unroll
           for (int t = 0; t < N; ++t) same = same || (fr.k[t] == key && (fr.v[t] & ~kExpanded) == id);
           if (__ballot(same) == 0ull) {
-            resume_at = j;  // an equal key of another node (WATCH: or a watched eviction): the rules for equal keys apply from this offer on
-            todo = 0ull;
+            if constexpr (BUILD) {
+              // the build takes equal keys as they come (order of arrival): any deterministic choice is as good
+              frontier_insert_distinct<NS>(fr, key, id);
+              st.n_acc = st.n_acc + 1;
+              if (!FULL && st.n_acc < ef) {
+                st.maxkey = uni(fmaxf(st.maxkey, key));
+                st.lower = st.maxkey;
+              } else {
+                st.lower = frontier_max<NS>(fr);
+              }
+            } else {
+              resume_at = j;  // an equal key of another node (WATCH: or a watched eviction): the rules for equal keys apply from this offer on
+              todo = 0ull;
+            }
           }
           // (else: a node met again after the visited filter forgot it; it is in the set already)
         }
@@ -1126,12 +1141,15 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   // instructions per accepted candidate — and only then moves on to the general loop below, at the very offer
   // that met the equal key (resume_at).
   int resume_at = -1;
-  bool calm = exact && S <= 64;  // no equal keys are at work: the tie-free loop may run
+  bool calm = (exact || (BUILD && !far)) && S <= 64;  // no equal keys are at work (or none matter): the tie-free loop may run
   TieWatch watch;
   while (true) {
   if (calm) {
     int how = st.n_acc >= ef ? 2 : 0;
-    if (!have_tie) {
+    if constexpr (BUILD) {
+      if (how == 0) how = tie_free_phase<DT, QR, NS, false, false, false, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+      if (how == 2) how = tie_free_phase<DT, QR, NS, true, false, false, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+    } else if (!have_tie) {
       if (how == 0) how = tie_free_phase<DT, QR, NS, false, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
       if (how == 2) how = tie_free_phase<DT, QR, NS, true, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
     } else {

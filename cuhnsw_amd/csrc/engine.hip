@@ -646,6 +646,7 @@ class Engine {
       if (side) {
         SearchArgs b = a;
         b.live = 1;
+        b.entry = in_order ? d_entry.p : nullptr;  // (a query reaches that pass after the batch's descents are done)
         b.counter = d_ctl.p + 96;
         b.pool = pool;
         // one or two of these wavefronts per CU: LDS for a candidate queue that never spills costs the first

@@ -101,13 +101,19 @@ __device__ __forceinline__ StageTree make_stage_tree(int lane) {
   return st;
 }
 
-// priority_queue::pop
+// priority_queue::pop.  libstdc++ moves the hole from the root down to a leaf, always into the larger child (the
+// right one when the two compare equal), and then lets the former last entry rise from there while its
+// parent is smaller.  On the way down every child moved up one level, and along that path the keys do not
+// grow: the entries the last one rises past are exactly the path's deepest ones that compare smaller, they end
+// up where they were, and nothing below the place the last entry lands in changes at all.  So the way down
+// stops at the first moved child that is smaller than the last entry, which is written there -- same array
+// as the two loops of libstdc++, one pass, no second look at the path.
 template <bool MINQ, class Acc>
 __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tree, int lane) {
   if (size > 1) {
     wave_sync();
     const int len = size - 1;
-    const HeapEnt value = uniform_ent(h.get(len));
+    const HeapEnt last_ent = h.get(len);  // (the same in every lane; its read travels with the first stage's)
     // lane t < 63 stands for the t-th node (breadth first) of the subtree under the hole
     const int d = 31 - __clz(lane + 1);
     const int o = lane + 1 - (1 << d);
@@ -117,7 +123,7 @@ __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tre
       const int c1 = 2 * P + 1;
       const bool has1 = lane < 63 && c1 < len;
       const bool has2 = lane < 63 && c1 + 1 < len;
-      HeapEnt L = value, R = value;
+      HeapEnt L = last_ent, R = last_ent;
       if (has1) {
         L = h.get(c1);
         R = h.get(c1 + 1);  // c1 + 1 <= len is a valid slot
@@ -133,18 +139,25 @@ __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tre
       const unsigned long long me = __ballot(edge);
       const bool on_path = lane < 63 && (me & tree.anc) == tree.anc;
       const unsigned long long mp = __ballot(on_path);
-      if (on_path && has1) h.set(P, take_left ? L : R);
+      const HeapEnt child = take_left ? L : R;
+      // path nodes whose chosen child is smaller than the last entry (deeper nodes have higher lane numbers)
+      const unsigned long long mr = __ballot(on_path && has1 && heap_less<MINQ>(child.key, last_ent.key));
+      if (mr != 0ull) {
+        const int first = __builtin_ctzll(mr);
+        if (on_path && lane <= first) h.set(P, lane < first ? child : last_ent);
+        break;
+      }
+      if (on_path && has1) h.set(P, child);
       const int last = 63 - __builtin_clzll(mp);  // deepest node of the path inside this stage
       const int dd = 31 - __clz(last + 1);
       const int last_abs = ((hole + 1) << dd) - 1 + (last + 1 - (1 << dd));
       if (((mc >> last) & 1ull) == 0ull) {
-        hole = last_abs;  // no child: the hole stops here
+        if (lane == last) h.set(P, last_ent);  // no child: the hole stops here, and so does the last entry
         break;
       }
       hole = 2 * last_abs + 2 - (int)((ml >> last) & 1ull);  // its chosen child roots the next stage
       wave_sync();
     }
-    coop_sift_up<MINQ>(h, hole, value, lane);
   }
   size = size - 1;
 }

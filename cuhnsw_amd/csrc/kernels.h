@@ -638,8 +638,17 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
     topkeys_init<NS>(tk, a.ef, lane);
 
     uint32_t cur = ix.enterpoint;
-    float dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
-    descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
+    float dcur;
+    if (a.entry) {  // the descent through the upper levels has been done for the whole batch
+      const uint4 en = a.entry[qi];
+      cur = (uint32_t)__builtin_amdgcn_readfirstlane((int)en.x);
+      dcur = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane((int)en.y));
+      st.n_dist_upper = __builtin_amdgcn_readfirstlane((int)en.z);
+      st.n_sweeps = __builtin_amdgcn_readfirstlane((int)en.w);
+    } else {
+      dcur = dist_single<DT, QR>(ix, qv, cur, s, lane);
+      descend<DT, QR>(ix, qv, ix.maxlevel, 0, cur, dcur, s, st, lane);
+    }
 
     int T;
     bool literal = NS == 0;

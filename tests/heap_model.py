@@ -67,6 +67,8 @@ def push_coop(a, size, v, minq=False):
 
 
 def pop_coop(a, size, minq=False):
+  """The way down and the last entry's way up again in one pass: the way down stops at the first moved child that
+  compares smaller than the last entry, which is written there; everything below stays as it was."""
   if size > 1:
     ln = size - 1
     value = a[ln]
@@ -93,13 +95,20 @@ def pop_coop(a, size, minq=False):
           t = par
         return True
       path = [t for t in range(63) if on_path(t)]
-      writes = [(pos[t], left[t] if take_left[t] else right[t]) for t in path if has1[t]]
+      child = {t: (left[t] if take_left[t] else right[t]) for t in path if has1[t]}
+      rising = [t for t in path if has1[t] and less(minq, child[t][0], value[0])]
+      if rising:
+        first = min(rising)
+        writes = [(pos[t], child[t] if t < first else value) for t in path if t <= first]
+        for slot, e in writes:
+          a[slot] = e
+        break
+      writes = [(pos[t], child[t]) for t in path if has1[t]]
       for slot, e in writes:
         a[slot] = e
       last = max(path)
       if not has1[last]:
-        hole = pos[last]
+        a[pos[last]] = value
         break
       hole = 2 * pos[last] + 2 - (1 if take_left[last] else 0)
-    _sift_up_coop(a, hole, value, minq)
   return size - 1

@@ -14,13 +14,13 @@ pytestmark = pytest.mark.skipif(shutil.which(kernel_report.HIPCC) is None, reaso
 
 # kernel -> (wavefronts per SIMD at least, scratch bytes per lane at most)
 LIMITS = {
-    "search_fast_kernel<dot,1,5>": (7, 64),
-    "search_fast_kernel<dot,1,5,trails>": (7, 64),
-    "search_fast_kernel<l2,1,5>": (7, 64),
-    "search_fast_kernel<dot,2,5>": (7, 88),
-    "search_fast_kernel<l2,2,5>": (7, 104),
-    "search_fast_kernel<l2,2,5,trails>": (7, 88),
-    "search_fast_kernel<dot,1,2>": (7, 20),
+    "search_fast_kernel<dot,1,5>": (7, 68),
+    "search_fast_kernel<dot,1,5,trails>": (7, 56),
+    "search_fast_kernel<l2,1,5>": (7, 60),
+    "search_fast_kernel<dot,2,5>": (7, 60),
+    "search_fast_kernel<l2,2,5>": (7, 88),
+    "search_fast_kernel<l2,2,5,trails>": (7, 76),
+    "search_fast_kernel<dot,1,2>": (7, 0),
     "search_fast_kernel<dot,2,8>": (5, 36),
 }
 
