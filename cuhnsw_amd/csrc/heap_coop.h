@@ -72,6 +72,9 @@ __device__ __forceinline__ void coop_sift_up(Acc& h, int i, HeapEnt v, int lane)
     const int slot = ((i + 1) >> lane) - 1;
     h.set(slot, lane < t ? e : v);
   }
+  // (the lanes meet again here: merged into a caller's join, the end of the some-lanes store above would make
+  // the caller's size count as lane-dependent, and with it every loop over the heap)
+  __builtin_amdgcn_wave_barrier();
 }
 
 // priority_queue::emplace
@@ -145,6 +148,7 @@ __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tre
       if (mr != 0ull) {
         const int first = __builtin_ctzll(mr);
         if (on_path && lane <= first) h.set(P, lane < first ? child : last_ent);
+        __builtin_amdgcn_wave_barrier();
         break;
       }
       if (on_path && has1) h.set(P, child);
@@ -153,6 +157,7 @@ __device__ __forceinline__ void coop_pop(Acc& h, int& size, const StageTree& tre
       const int last_abs = ((hole + 1) << dd) - 1 + (last + 1 - (1 << dd));
       if (((mc >> last) & 1ull) == 0ull) {
         if (lane == last) h.set(P, last_ent);  // no child: the hole stops here, and so does the last entry
+        __builtin_amdgcn_wave_barrier();
         break;
       }
       hole = 2 * last_abs + 2 - (int)((ml >> last) & 1ull);  // its chosen child roots the next stage
