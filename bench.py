@@ -38,11 +38,15 @@ KERNEL_SOURCES = ["device_core.h", "heap_coop.h", "kernels.h", "engine.hip"]
 
 
 def kernel_source_digest():
-  """Digest of the kernel sources: a traffic figure measured on other kernels is not reported."""
+  """Digest of the kernel sources without their comments and blank space: a traffic figure measured on other
+  kernels is not reported."""
   h = hashlib.sha256()
   for name in KERNEL_SOURCES:
-    with open(os.path.join(ROOT, "cuhnsw_amd", "csrc", name), "rb") as f:
-      h.update(f.read())
+    with open(os.path.join(ROOT, "cuhnsw_amd", "csrc", name), "r") as f:
+      for line in f:
+        code = line.split("//", 1)[0].strip()
+        if code:
+          h.update(" ".join(code.split()).encode() + b"\n")
   return h.hexdigest()[:16]
 
 

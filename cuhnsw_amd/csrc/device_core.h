@@ -993,9 +993,13 @@ __device__ __forceinline__ void trail_stop(Trail& tr, int hops, int n_dist) {
 // FULL = true: the set holds ef entries (the bound is its last key, an accepted offer pushes one out) — two
 // instantiations, so that the hot one carries neither the fill test nor the running maximum.  TRAILS: the hop's
 // accepted entries go on the search's trail (a kernel instance of its own: a pass that keeps no trails pays
-// nothing for them).  Returns 0: no waiting entry is left, the search is over; 1: an
-// offer met an equal key of another node (resume_at = which offer of the list in s.nbuf / s.dbuf); 2 (FULL = false
-// only): the set is full now, the other phase goes on.  n = ids waiting in s.nbuf on entry.
+// nothing for them).  WATCH: the set holds equal keys that do no harm as long as the waiting entries on the watch
+// list (those with an equal in the set) are neither expanded nor pushed out here -- the loop hands back to the
+// general one when that is about to happen.  BUILD: equal keys are taken in order of arrival and nothing is ever
+// handed back.  Returns 0: no waiting entry is left, the search is over; 1: an offer met an equal key of another
+// node, or its eviction would reach a watched entry (resume_at = which offer of the list in s.nbuf / s.dbuf);
+// 2 (FULL = false only): the set is full now, the other phase goes on; 3 (WATCH only): the next candidate is a
+// watched entry (its expanded mark has been taken off again, n = 0).  n = ids waiting in s.nbuf on entry.
 template <int DT, int QR, int NS, bool FULL, bool TRAILS, bool WATCH, bool BUILD = false>
 __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, int S, Scratch& s,
                                               SearchState& st, Frontier<NS>& fr, int& n, int& hop_cid, int& resume_at,
