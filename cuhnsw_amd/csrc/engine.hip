@@ -605,11 +605,12 @@ class Engine {
       // A handed-over query is not searched again from its entry point: the first pass leaves the entries it
       // accepted, hop by hop, and the literal pass (on the sorted set with ids: it needs no visited bitmap
       // brought up to date) replays its queue operations from them up to where the two may part.  One query per
-      // wavefront, link rows of one pass of 64 lanes, and batches of up to two rounds of wavefronts: keeping the
-      // trail costs the first pass 2 to 3 %, which only a batch short enough to wait for its last hand-over
-      // gets back.  trails = 2: whatever the batch.
+      // wavefront, link rows of one pass of 64 lanes, and batches of under three rounds of wavefronts: keeping
+      // the trail costs the first pass 9 % (the kernel instance with the trail code 4 %, writing the records the
+      // rest), which only a batch short enough to wait for its last hand-over gets back.  trails = 2: whatever
+      // the batch.
       bool keep_trails = (QR == 1 || QR == 2) && trails && !a.reverse && a.lean && host.S0 <= 63 &&
-                         (trails > 1 || a.nq <= 2 * resident);
+                         (trails > 1 || 4 * (long long)a.nq <= 11 * resident);
       if (keep_trails) {
         // (normally there since the index became resident; a changed trail_cap / trail_spares asks again)
         if (d_trail.n < trail_records_wanted(slots)) {

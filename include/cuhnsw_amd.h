@@ -210,7 +210,7 @@ int cuhnsw_trails_available(cuhnsw_engine* e);
  *                   128 elements; 270 MB of device memory for 2048 accepted entries per query at work,
  *                   allocated when the index becomes resident (build_graph, load_index) — if that memory is
  *                   not there, searches go on without trails (cuhnsw_trails_available).  Keeping
- *                   the trail costs the first pass 2 to 3 %: 1 (default) = for batches of up to two rounds of
+ *                   the trail costs the first pass 9 %: 1 (default) = for batches of under three rounds of
  *                   wavefronts, which wait for their last hand-over; 2 = for every batch; 0 = off.
  *   "trail_cap"     accepted entries a trail holds (default 2048; a search that accepts more leaves none)
  *   "trail_spares"  handed-over queries per batch that can come with a trail (default 1024: each keeps the
