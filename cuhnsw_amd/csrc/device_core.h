@@ -1148,172 +1148,172 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
   bool calm = (exact || (BUILD && !far)) && S <= 64;  // no equal keys are at work (or none matter): the tie-free loop may run
   TieWatch watch;
   while (true) {
-  if (calm) {
-    int how = st.n_acc >= ef ? 2 : 0;
-    if constexpr (BUILD) {
-      if (how == 0) how = tie_free_phase<DT, QR, NS, false, false, false, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
-      if (how == 2) how = tie_free_phase<DT, QR, NS, true, false, false, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
-    } else if (!have_tie) {
-      if (how == 0) how = tie_free_phase<DT, QR, NS, false, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
-      if (how == 2) how = tie_free_phase<DT, QR, NS, true, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
-    } else {
-      // (after equal keys have met, the tie-free loop takes over again only once the set is full: how == 2)
-      how = tie_free_phase<DT, QR, NS, true, TRAILS, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
-    }
-    st.top_size = st.n_acc < ef ? st.n_acc : ef;
-    if (how == 0) {
-      trail_stop(tr, st.n_hops, st.n_dist);
-      return have_tie ? 2 : 0;
-    }
-    calm = false;
-    // (what these were when the tie-free loop took over; said again so that none of them has to live through it)
-    ghosts = 0;
-    ghost = kEmpty;
-    twin_phase = false;
-    in_group = false;
-    group_key = 0.f;
-    group_edge = INFINITY;
-    ek_min = INFINITY;
-    gave_up = false;
-  }
-  while (true) {
-    if (resume_at < 0) {
-      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
-      st.n_dist += n;
-      wave_sync();
-    }
-    for (int base = 0; base < n; base += 64) {
-      const int mine = base + lane;
-      // unconditional LDS reads at a clamped index, then a select: no exec-mask branches
-      const int at = mine < n ? mine : 0;
-      const float my_key = mine < n ? s.dbuf[at] : INFINITY;
-      const uint32_t my_id = s.nbuf[at];
-      const bool pass = mine < n && (st.n_acc < ef || st.lower > my_key);
-      unsigned long long todo = __ballot(pass);
-      if (resume_at >= 0) {
-        todo &= ~((1ull << resume_at) - 1ull);  // the offers before it have been dealt with (one list of at most 64)
-        resume_at = -1;
+    if (calm) {
+      int how = st.n_acc >= ef ? 2 : 0;
+      if constexpr (BUILD) {
+        if (how == 0) how = tie_free_phase<DT, QR, NS, false, false, false, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+        if (how == 2) how = tie_free_phase<DT, QR, NS, true, false, false, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+      } else if (!have_tie) {
+        if (how == 0) how = tie_free_phase<DT, QR, NS, false, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+        if (how == 2) how = tie_free_phase<DT, QR, NS, true, TRAILS, false>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
+      } else {
+        // (after equal keys have met, the tie-free loop takes over again only once the set is full: how == 2)
+        how = tie_free_phase<DT, QR, NS, true, TRAILS, true>(ix, qv, level, ef, S, s, st, fr, n, hop_cid, resume_at, accepted, tr, watch, lane);
       }
-      // offers turned away while a group of equal keys is being expanded: remember the closest
-      if (exact && in_group) group_edge = uni(fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY)));
-      // (plain if/else nesting, one way out of the loop: `continue` and `return` in here make the
-      // compiler thread a state variable through a dozen scalar blocks per accepted candidate)
-      while (todo != 0ull) {
-        const int j = __builtin_ctzll(todo);
-        todo &= todo - 1ull;
-        const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
-        const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
-        if (st.n_acc < ef || st.lower > key) {
-          // an eviction out of several equal largest keys: the heap's choice decides which of
-          // them stays in the result set, and the other one stays a live candidate of hnswlib
-          const bool twins = exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr);
-          // the entry a full set is about to push out, where somebody will ask for it
-          const uint32_t evicted = (twins || (exact && in_group && st.n_acc >= ef && st.lower == group_key))
-                                       ? (uint32_t)__builtin_amdgcn_readlane((int)fr.v[(NS > 0 ? NS : 1) - 1], 63)
-                                       : kEmpty;
-          const int r = frontier_insert<NS>(fr, key, id, lane);
-          if (r != 2) {
-            accepted |= 1ull << j;
-            if (twins) {
-              ek_min = uni(fminf(ek_min, st.lower));
-              ghost = evicted;
-              // (three or more equal largest keys, a second event, the whole set asked for: the plain rule)
-              ghosts += (frontier_max_twice<NS>(fr) || whole_set) ? 2 : 1;
-            }
-            if (exact && twin_phase) {
-              gave_up = true;  // which twin hnswlib expands first now decides whether the other one is expanded at all
-              todo = 0ull;
-            }
-            have_tie = have_tie || r == 1;
-            if (exact && in_group && st.n_acc >= ef) {
-              group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
-              // a member of the group pushed out before its turn: with another order it would have been expanded
-              if (st.lower == group_key && (evicted & kExpanded) == 0u) {
-                gave_up = true;
+      st.top_size = st.n_acc < ef ? st.n_acc : ef;
+      if (how == 0) {
+        trail_stop(tr, st.n_hops, st.n_dist);
+        return have_tie ? 2 : 0;
+      }
+      calm = false;
+      // (what these were when the tie-free loop took over; said again so that none of them has to live through it)
+      ghosts = 0;
+      ghost = kEmpty;
+      twin_phase = false;
+      in_group = false;
+      group_key = 0.f;
+      group_edge = INFINITY;
+      ek_min = INFINITY;
+      gave_up = false;
+    }
+    while (true) {
+      if (resume_at < 0) {
+        if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+        st.n_dist += n;
+        wave_sync();
+      }
+      for (int base = 0; base < n; base += 64) {
+        const int mine = base + lane;
+        // unconditional LDS reads at a clamped index, then a select: no exec-mask branches
+        const int at = mine < n ? mine : 0;
+        const float my_key = mine < n ? s.dbuf[at] : INFINITY;
+        const uint32_t my_id = s.nbuf[at];
+        const bool pass = mine < n && (st.n_acc < ef || st.lower > my_key);
+        unsigned long long todo = __ballot(pass);
+        if (resume_at >= 0) {
+          todo &= ~((1ull << resume_at) - 1ull);  // the offers before it have been dealt with (one list of at most 64)
+          resume_at = -1;
+        }
+        // offers turned away while a group of equal keys is being expanded: remember the closest
+        if (exact && in_group) group_edge = uni(fminf(group_edge, wave_min((mine < n && !pass) ? my_key : INFINITY)));
+        // (plain if/else nesting, one way out of the loop: `continue` and `return` in here make the
+        // compiler thread a state variable through a dozen scalar blocks per accepted candidate)
+        while (todo != 0ull) {
+          const int j = __builtin_ctzll(todo);
+          todo &= todo - 1ull;
+          const float key = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_key), j));
+          const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, j);
+          if (st.n_acc < ef || st.lower > key) {
+            // an eviction out of several equal largest keys: the heap's choice decides which of
+            // them stays in the result set, and the other one stays a live candidate of hnswlib
+            const bool twins = exact && have_tie && st.n_acc >= ef && frontier_max_twice<NS>(fr);
+            // the entry a full set is about to push out, where somebody will ask for it
+            const uint32_t evicted = (twins || (exact && in_group && st.n_acc >= ef && st.lower == group_key))
+                                         ? (uint32_t)__builtin_amdgcn_readlane((int)fr.v[(NS > 0 ? NS : 1) - 1], 63)
+                                         : kEmpty;
+            const int r = frontier_insert<NS>(fr, key, id, lane);
+            if (r != 2) {
+              accepted |= 1ull << j;
+              if (twins) {
+                ek_min = uni(fminf(ek_min, st.lower));
+                ghost = evicted;
+                // (three or more equal largest keys, a second event, the whole set asked for: the plain rule)
+                ghosts += (frontier_max_twice<NS>(fr) || whole_set) ? 2 : 1;
+              }
+              if (exact && twin_phase) {
+                gave_up = true;  // which twin hnswlib expands first now decides whether the other one is expanded at all
                 todo = 0ull;
               }
+              have_tie = have_tie || r == 1;
+              if (exact && in_group && st.n_acc >= ef) {
+                group_edge = uni(fminf(group_edge, st.lower));  // the entry this insert evicted
+                // a member of the group pushed out before its turn: with another order it would have been expanded
+                if (st.lower == group_key && (evicted & kExpanded) == 0u) {
+                  gave_up = true;
+                  todo = 0ull;
+                }
+              }
+              st.n_acc = uni(st.n_acc + 1);
+              st.maxkey = uni(fmaxf(st.maxkey, key));
+              st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
             }
-            st.n_acc = uni(st.n_acc + 1);
-            st.maxkey = uni(fmaxf(st.maxkey, key));
-            st.lower = uni(st.n_acc >= ef ? frontier_max<NS>(fr) : st.maxkey);  // hnswlib's lowerBound
+          } else if (exact && in_group) {
+            group_edge = uni(fminf(group_edge, key));
           }
-        } else if (exact && in_group) {
-          group_edge = uni(fminf(group_edge, key));
         }
+        if (gave_up) base = n;  // leave the outer loop as well
+        else trail_hop(tr, accepted, hop_cid, st.n_hops, my_id, my_key, lane);  // (a trail is kept for rows of one pass only)
+        accepted = 0ull;
       }
-      if (gave_up) base = n;  // leave the outer loop as well
-      else trail_hop(tr, accepted, hop_cid, st.n_hops, my_id, my_key, lane);  // (a trail is kept for rows of one pass only)
-      accepted = 0ull;
-    }
-    if (gave_up) {
-      trail_stop(tr, st.n_hops - 1, st.n_dist - n);  // (a trail still recording here: the hop under way, and its evaluations, are not on it)
-      break;
-    }
-    st.top_size = st.n_acc < ef ? st.n_acc : ef;
-    int cid = frontier_take<NS>(fr, lane, far);
-    const bool was_in_group = in_group;
-    if (exact && have_tie) {
-      const float d = cid >= 0 ? frontier_key_of<NS>(fr, (uint32_t)cid) : INFINITY;
-      if (in_group && cid >= 0 && d < group_key) {
-        // a closer candidate turned up inside the group: it is expanded before the rest of the group under any
-        // order.  A group within the group is not followed.
-        gave_up = frontier_open_key<NS>(fr, d);
-      } else if (in_group && d != group_key) {
-        // the group is through.  With another order of its members an offer or an entry whose
-        // key equals the bound reached now could have ended up on the other side of it; and with the bound
-        // below the group's key a member popped late would not have been expanded at all.
-        gave_up = st.n_acc >= ef && (group_edge == st.lower || st.lower < group_key);
-        in_group = false;
+      if (gave_up) {
+        trail_stop(tr, st.n_hops - 1, st.n_dist - n);  // (a trail still recording here: the hop under way, and its evaluations, are not on it)
+        break;
       }
-      if (cid >= 0) {
-        if (d >= ek_min) {
-          // the twin the set kept: it is the set's last entry and its key is the bound
-          if (ghosts == 1 && !in_group && !frontier_open_key<NS>(fr, d)) twin_phase = true;
-          else gave_up = true;
+      st.top_size = st.n_acc < ef ? st.n_acc : ef;
+      int cid = frontier_take<NS>(fr, lane, far);
+      const bool was_in_group = in_group;
+      if (exact && have_tie) {
+        const float d = cid >= 0 ? frontier_key_of<NS>(fr, (uint32_t)cid) : INFINITY;
+        if (in_group && cid >= 0 && d < group_key) {
+          // a closer candidate turned up inside the group: it is expanded before the rest of the group under any
+          // order.  A group within the group is not followed.
+          gave_up = frontier_open_key<NS>(fr, d);
+        } else if (in_group && d != group_key) {
+          // the group is through.  With another order of its members an offer or an entry whose
+          // key equals the bound reached now could have ended up on the other side of it; and with the bound
+          // below the group's key a member popped late would not have been expanded at all.
+          gave_up = st.n_acc >= ef && (group_edge == st.lower || st.lower < group_key);
+          in_group = false;
         }
-        if (!in_group && !twin_phase) {
-          in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
-          group_key = d;
-          group_edge = INFINITY;
-        }
-      } else if (!gave_up && st.n_acc >= ef && st.lower >= ek_min) {
-        // an entry evicted out of equal largest keys that are still within the bound is one
-        // hnswlib would go on to expand
-        if (ghosts == 1) {
-          if ((ghost & kExpanded) == 0u) {
-            cid = (int)ghost;  // the twin the set pushed out: expanded like any other, nothing of it may be accepted
-            ghost |= kExpanded;
-            twin_phase = true;
+        if (cid >= 0) {
+          if (d >= ek_min) {
+            // the twin the set kept: it is the set's last entry and its key is the bound
+            if (ghosts == 1 && !in_group && !frontier_open_key<NS>(fr, d)) twin_phase = true;
+            else gave_up = true;
           }
-        } else {
-          gave_up = true;
+          if (!in_group && !twin_phase) {
+            in_group = frontier_open_key<NS>(fr, d);  // other waiting entries with this very key
+            group_key = d;
+            group_edge = INFINITY;
+          }
+        } else if (!gave_up && st.n_acc >= ef && st.lower >= ek_min) {
+          // an entry evicted out of equal largest keys that are still within the bound is one
+          // hnswlib would go on to expand
+          if (ghosts == 1) {
+            if ((ghost & kExpanded) == 0u) {
+              cid = (int)ghost;  // the twin the set pushed out: expanded like any other, nothing of it may be accepted
+              ghost |= kExpanded;
+              twin_phase = true;
+            }
+          } else {
+            gave_up = true;
+          }
         }
       }
+      // the trail: over for good, or the hops of a group of equal keys begin or end with the next one
+      if (twin_phase || gave_up || cid < 0) trail_stop(tr, st.n_hops, st.n_dist);
+      else if (in_group != was_in_group) trail_mark(tr, in_group ? kTrailOwn : kTrailBack, st.n_hops + 1, lane);
+      if (gave_up || cid < 0) break;
+      hop_cid = cid;
+      st.n_hops += 1;
+      wave_sync();
+      n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
+      wave_sync();
+      // Equal keys that sit in the set do no harm while none of them that still waits is expanded or pushed out
+      // (unless the whole set is the answer): no group can form, and which of two expanded twins an eviction
+      // pushes out changes neither the keys of the set nor hnswlib's candidates.  With no group under way and
+      // no eviction out of equal largest keys on record whose key is still within the bound (once the bound is
+      // below it, the entry such an eviction pushed out is as dead for hnswlib as any other), the tie-free loop
+      // takes over again from this hop's offers, with the waiting entries that have an equal (at most four) on
+      // its watch list; it comes back at the next offer that meets an equal key, when a watched entry's turn
+      // comes, or when an eviction reaches one.
+      if (exact && S <= 64 && !whole_set && st.n_acc >= ef && !in_group && !twin_phase && (ghosts == 0 || st.lower < ek_min) &&
+          frontier_watch_list<NS>(fr, watch)) {
+        calm = true;
+        break;
+      }
     }
-    // the trail: over for good, or the hops of a group of equal keys begin or end with the next one
-    if (twin_phase || gave_up || cid < 0) trail_stop(tr, st.n_hops, st.n_dist);
-    else if (in_group != was_in_group) trail_mark(tr, in_group ? kTrailOwn : kTrailBack, st.n_hops + 1, lane);
-    if (gave_up || cid < 0) break;
-    hop_cid = cid;
-    st.n_hops += 1;
-    wave_sync();
-    n = visit_lossy(link_row(ix, (uint32_t)cid, level), S, s, lane);
-    wave_sync();
-    // Equal keys that sit in the set do no harm while none of them that still waits is expanded or pushed out
-    // (unless the whole set is the answer): no group can form, and which of two expanded twins an eviction
-    // pushes out changes neither the keys of the set nor hnswlib's candidates.  With no group under way and
-    // no eviction out of equal largest keys on record whose key is still within the bound (once the bound is
-    // below it, the entry such an eviction pushed out is as dead for hnswlib as any other), the tie-free loop
-    // takes over again from this hop's offers, with the waiting entries that have an equal (at most four) on
-    // its watch list; it comes back at the next offer that meets an equal key, when a watched entry's turn
-    // comes, or when an eviction reaches one.
-    if (exact && S <= 64 && !whole_set && st.n_acc >= ef && !in_group && !twin_phase && (ghosts == 0 || st.lower < ek_min) &&
-        frontier_watch_list<NS>(fr, watch)) {
-      calm = true;
-      break;
-    }
-  }
-  if (!calm) break;
+    if (!calm) break;
   }
   return gave_up ? 1 : (have_tie ? 2 : 0);
 }
