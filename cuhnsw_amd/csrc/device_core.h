@@ -870,6 +870,76 @@ __device__ __forceinline__ void frontier_dump(const Frontier<NS>& f, int ef, int
   }
 }
 
+// The reference's reverse_cand search (expand the farthest waiting candidate, GetCand(..., reverse),
+// cpp/include/cuda_utils_kernels.cuh:104-151) for result sets beyond the register set's capacity: one sorted list in
+// LDS (s.top, ef entries, ascending; bit 31 of the id = expanded), equal keys in order of arrival, the last entry
+// leaves a full list.  An insert counts the keys not above the new one (the list is sorted: whole chunks of 64
+// until the first that is not) and moves the tail up one place, 64 entries at a time from the top; the next
+// candidate is the last entry without the mark.  Exact visited bitmap.  A list of a thousand entries makes an
+// insert a few dozen LDS round trips: the option is there for completeness, not for speed.  On entry
+// s.nbuf[0..n_seed) holds the seeds (marked visited); on exit s.top[0..st.top_size) is the result in order.
+template <int DT, int QR>
+__device__ __forceinline__ void search_level_far_lds(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
+                                                     SearchState& st, int n_seed, int lane) {
+  HeapEnt* set = s.top;
+  const int S = row_stride(ix, level);
+  int size = 0;
+  int n = n_seed;
+  while (true) {
+    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    st.n_dist += n;
+    wave_sync();
+    for (int j = 0; j < n; ++j) {
+      const float key = s.dbuf[j];   // (the same address in every lane)
+      const uint32_t id = s.nbuf[j];
+      const float last_key = size > 0 ? set[size - 1].key : INFINITY;
+      if (size < ef || last_key > key) {
+        // where it goes: after every entry whose key is not above it
+        int p = 0;
+        for (int base = 0; base < size; base += 64) {
+          const int i = base + lane;
+          const unsigned long long le = __ballot(i < size && set[i < size ? i : 0].key <= key);
+          p += __popcll(le);
+          if (__popcll(le) < (size - base < 64 ? size - base : 64)) break;
+        }
+        const int new_size = size < ef ? size + 1 : ef;
+        // entries [p, new_size - 1) move up one place, the topmost chunk first (each chunk is read whole
+        // before it is written)
+        for (int hi = new_size - 1; hi > p; hi -= 64) {
+          const int dst = hi - lane;
+          HeapEnt e = set[dst > p ? dst - 1 : p];
+          wave_sync();
+          if (dst > p) set[dst] = e;
+          wave_sync();
+        }
+        if (lane == 0) {
+          HeapEnt e;
+          e.key = key;
+          e.id = id;
+          set[p] = e;
+        }
+        wave_sync();
+        size = new_size;
+      }
+    }
+    // the farthest entry still waiting
+    int pick = -1;
+    for (int hi = size - 1; hi >= 0 && pick < 0; hi -= 64) {
+      const int i = hi - lane;
+      const unsigned long long open = __ballot(i >= 0 && (set[i >= 0 ? i : 0].id & kExpanded) == 0u);
+      if (open != 0ull) pick = hi - __builtin_ctzll(open);
+    }
+    if (pick < 0) break;
+    const uint32_t cid = set[pick].id;
+    wave_sync();
+    if (lane == 0) set[pick].id = cid | kExpanded;
+    st.n_hops += 1;
+    n = visit_row(link_row(ix, cid, level), S, s, st, lane);
+    wave_sync();
+  }
+  st.top_size = size;
+}
+
 // The sorted-set search's visited filter: a four-way set-associative tag cache in LDS alone, no
 // bitmap.  A set is one 64-bit word holding four 16-bit tags (set = low id bits, tag = the
 // rest; 0xFFFF = empty); a new tag pushes the oldest of the four out.  A hit is exact ("seen

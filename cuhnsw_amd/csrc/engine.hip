@@ -865,10 +865,13 @@ class Engine {
     a.vc_bits = auto_vc_bits();
     a.fast_path = no_alloc ? 2 : (fast_suspended ? 0 : fast_path);
     a.reverse = opt.reverse_cand ? 1 : 0;
-    if (a.reverse) a.fast_path = 2;  // only the sorted set can expand its farthest entry
+    // reverse_cand: the sorted set in registers expands its farthest entry; beyond its capacity (ef >= 1024) the
+    // literal pass does, on a sorted list in LDS
+    if (a.reverse) a.fast_path = ns > 0 ? 2 : 0;
+    if (a.reverse && no_alloc && ns == 0) throw std::runtime_error("search_knn (no allocation): reverse_cand needs ef_search below 1024");
     a.fc_bits = (ns > 0 && a.fast_path) ? auto_fc_bits(ef) : 0;
-    if (a.reverse && a.fc_bits == 0)
-      throw std::runtime_error("search_knn: reverse_cand needs ef_search below 1024 and fewer than 2^28 points");
+    if (a.reverse && ns > 0 && a.fc_bits == 0)
+      throw std::runtime_error("search_knn: reverse_cand needs fewer than 2^28 points");
     // with the keys in registers the queue's LDS share doubles as result buffer (lcap entries,
     // then lcap label slots) and as the replay heap (ef + 1 entries)
     const int floor_entries = ns > 0 ? std::max(ef + 1, 2 * a.lcap) : std::max(k, 64);

@@ -739,6 +739,21 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
         st.top_size = size;
       }
       }
+    } else if (NS == 0 && a.reverse) {
+      // reverse_cand beyond the register set's capacity: a sorted list in LDS; the answer is its first k entries
+      vcache_reset(s, lane);
+      visit_single(s, st, cur, lane);
+      if (lane == 0) s.nbuf[0] = cur;
+      wave_sync();
+      search_level_far_lds<DT, QR>(ix, qv, 0, a.ef, s, st, 1, lane);
+      literal = false;
+      T = st.top_size < a.k ? st.top_size : a.k;
+      wave_sync();
+      for (int e = lane; e < T; e += 64) {  // (the list has its own LDS: NS == 0)
+        s.nbuf[e] = s.top[e].id & ~kExpanded;
+        s.dbuf[e] = s.top[e].key;
+      }
+      have_result = true;
     } else {
     vcache_reset(s, lane);
     visit_single(s, st, cur, lane);
