@@ -157,6 +157,7 @@ class Engine {
 
   // tunables
   int level_first = 1;     // build: a batch hands out its nodes with upper levels first
+  int build_literal = 0;   // build: 1 = the literal search (queues / sorted list in LDS) whatever ef_construction (tests)
   int build_batch = 0;     // nodes inserted per batch at most; 0 = by the size of the graph (batch_at)
   int search_slots = 0;
   int cand_lds_override = 0;
@@ -971,8 +972,7 @@ class Engine {
                    (QR == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
     a.fc_bits = NS > 0 ? auto_fc_bits(efc) : 0;
     const bool sorted_set = NS > 0 && a.fc_bits > 0;  // then neither queue nor literal cache is needed
-    if (a.reverse && !sorted_set)
-      throw std::runtime_error("build_graph: reverse_cand needs ef_construction below 1024 and fewer than 2^28 points");
+    if (a.reverse && NS > 0 && !sorted_set) throw std::runtime_error("build_graph: reverse_cand needs fewer than 2^28 points");
     a.cand_lds = sorted_set ? 0 : auto_cand_lds(efc, NS, 64, fixed);
     a.vc_bits = sorted_set ? 0 : auto_vc_bits();
     const LdsPlan lp1 = plan_lds(QR, Dp, sorted_set ? -1 : efc, a.cand_lds, a.lcap, efc, m_max, a.vc_bits, a.fc_bits);
@@ -1094,7 +1094,7 @@ class Engine {
     HIP_CHECK(hipStreamSynchronize(stream));
     auto t0 = std::chrono::steady_clock::now();
     const int q = qr();
-    const int ns = key_slots(opt.ef_construction);
+    const int ns = build_literal ? 0 : key_slots(opt.ef_construction);
     if (dist_type == DIST_DOT) build_qr<DIST_DOT>(q, ns);
     else build_qr<DIST_L2>(q, ns);
     last_build_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
@@ -1278,6 +1278,7 @@ int cuhnsw_set_tunable(cuhnsw_engine* e, const char* name, double value) {
   std::string n(name);
   if (n == "build_batch") e->impl.build_batch = (int)value;
   else if (n == "level_first") e->impl.level_first = (int)value;
+  else if (n == "build_literal") e->impl.build_literal = (int)value;
   else if (n == "search_slots") e->impl.search_slots = (int)value;
   else if (n == "cand_lds") e->impl.cand_lds_override = (int)value;
   else if (n == "hnswlib_dist") e->impl.hnswlib_dist = (int)value;

@@ -1010,6 +1010,21 @@ __global__ void __launch_bounds__(64, (NS <= 5 && QR == 1) ? 6 : ((NS <= 5 && QR
           wave_sync();
           frontier_dump<NS>(fr, a.efc, T, sid, skey, lane);
           wave_sync();
+        } else if (NS == 0 && a.reverse) {
+          // reverse_cand beyond the register set's capacity: a sorted list in LDS, already in order
+          vcache_reset(s, lane);
+          visit_single(s, st, x, lane);  // a node never links to itself
+          visit_single(s, st, cur, lane);
+          if (lane == 0) s.nbuf[0] = cur;
+          wave_sync();
+          search_level_far_lds<DT, QR>(ix, qv, level, a.efc, s, st, 1, lane);
+          T = st.top_size;
+          wave_sync();
+          for (int e = lane; e < T; e += 64) {
+            sid[e] = s.top[e].id & ~kExpanded;
+            skey[e] = s.top[e].key;
+          }
+          wave_sync();
         } else {
           vcache_reset(s, lane);
           visit_single(s, st, x, lane);  // a node never links to itself

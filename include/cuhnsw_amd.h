@@ -171,6 +171,9 @@ int cuhnsw_trails_available(cuhnsw_engine* e);
  *                   of the nodes already in, at most 16384; beyond 524288 nodes a thirty-second, at most 65536)
  *   "level_first"   1 (default) = a build batch hands out its nodes with upper levels first (they take several
  *                   searches each, and a launch ends when its last node does); 0 = by id.  Same graph either way.
+ *   "build_literal" 1 = the build searches with the literal structures in LDS (two priority queues, or the
+ *                   sorted list of reverse_cand) whatever ef_construction — what it does by itself from
+ *                   ef_construction 1024 on; same graph as with the sorted set in registers (a testing aid)
  *   "search_slots"  resident wavefronts used by search (0 = automatic)
  *   "cand_lds"      candidate-queue entries kept in LDS (0 = automatic)
  *   "hnswlib_dist"  1 = return hnswlib distances (1-dot) instead of -dot

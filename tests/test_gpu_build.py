@@ -283,3 +283,39 @@ def test_build_with_reverse_cand(oracle, tmp_path):
     ids, _, _ = ix.search(q, 10, 100)         # plain hnswlib search on both graphs
     rec[rev] = recall(ids, gt)
   assert rec[True] >= rec[False] - 0.01 and rec[True] >= 0.8, rec
+
+
+def test_reverse_cand_build_on_the_sorted_list_in_lds(oracle, tmp_path):
+  """From ef_construction 1024 on the reverse_cand build keeps its candidates in a sorted list in LDS instead of the
+  sorted set in registers.  Same rule, so the same graph: forced at a small ef_construction (tunable build_literal)
+  the file equals the register path's byte for byte; at ef_construction 1100 the graph is valid and searchable."""
+  import hashlib
+  n, d = 6000, 24
+  x = gauss_mixture(n, d, centres=60, seed=71)
+  mult = 1.0 / np.log(8)
+  levels = _levels(n, mult, 73)
+  digests = []
+  for forced in (0, 1):
+    from cuhnsw_amd import capi
+    e = capi.Engine()
+    path, _ = write_options(tmp_path, dist_type="l2", max_m=8, max_m0=16, ef_construction=80, heuristic_coef=0.0,
+                            reverse_cand=True)
+    assert e.init(path) == 0
+    e.set_tunable("build_literal", forced)
+    e.set_data(x)
+    e.set_random_levels(levels)
+    e.build_graph()
+    p = str(tmp_path / ("lds%d.idx" % forced))
+    e.save_index(p)
+    digests.append(hashlib.sha256(open(p, "rb").read()).hexdigest())
+  assert digests[0] == digests[1]
+  e = _build(tmp_path, x, levels, dist_type="l2", max_m=8, max_m0=16, ef_construction=1100, heuristic_coef=0.0,
+             reverse_cand=True)
+  p = str(tmp_path / "lds_big.idx")
+  e.save_index(p)
+  ix = oracle.OracleIndex("l2").load(p)
+  assert ix.validate() == 0
+  q = gauss_mixture(200, d, centres=60, seed=72)
+  gt, _ = oracle.bruteforce(x, q, 10, "l2")
+  ids, _, _ = ix.search(q, 10, 100)
+  assert recall(ids, gt) >= 0.9
