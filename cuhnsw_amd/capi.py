@@ -19,6 +19,7 @@ SYMBOLS = [
     "cuhnsw_search_knn_device_noalloc", "cuhnsw_last_build_dropped_links", "cuhnsw_debug_link_keys0",
     "cuhnsw_last_build_counters", "cuhnsw_debug_gather_probe", "cuhnsw_last_search_trails",
     "cuhnsw_last_search_side_by_side", "cuhnsw_literal_fallbacks", "cuhnsw_trails_available",
+    "cuhnsw_num_deleted",
 ]
 
 _lib = None
@@ -61,6 +62,7 @@ def load():
   l.cuhnsw_last_search_side_by_side.argtypes = [vp]
   l.cuhnsw_literal_fallbacks.argtypes = [vp]
   l.cuhnsw_trails_available.argtypes = [vp]
+  l.cuhnsw_num_deleted.argtypes = [vp]
   l.cuhnsw_set_tunable.argtypes = [vp, ctypes.c_char_p, cd]
   _lib = l
   return l
@@ -178,6 +180,7 @@ class Engine:
   num_dims = property(lambda s: s._l.cuhnsw_num_dims(s._h))
   max_level = property(lambda s: s._l.cuhnsw_max_level(s._h))
   enter_point = property(lambda s: s._l.cuhnsw_enter_point(s._h))
+  num_deleted = property(lambda s: s._l.cuhnsw_num_deleted(s._h))
   last_build_seconds = property(lambda s: s._l.cuhnsw_last_build_seconds(s._h))
   last_search_repeats = property(lambda s: s._l.cuhnsw_last_search_repeats(s._h))
   last_search_trails = property(lambda s: s._l.cuhnsw_last_search_trails(s._h))

@@ -532,8 +532,12 @@ __device__ __forceinline__ float topkeys_at(const TopKeys<NS>& t, int pos, int e
 // reference's, cpp/include/cuda_utils_kernels.cuh:220-225).  Wavefront-uniform: every lane
 // runs it, the heap moves are cooperative.  NS > 0: result keys in registers (TopKeys);
 // NS == 0: literal result heap in LDS (s.top), for ef beyond the register capacity.
+// deleted (NS == 0 only): one bit per element, hnswlib's delete marks (hnswlib searchBaseLayerST, has_deletions):
+// a marked element is queued as a candidate like any other and never enters the result heap; the bound moves
+// only while that heap holds something.
 template <int NS>
-__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys<NS>& tk, int n, int ef, int lane) {
+__device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys<NS>& tk, int n, int ef, int lane,
+                                            const uint32_t* deleted = nullptr) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int cand_cap = s.cand_lds + s.cand_glob_cap;
   for (int base = 0; base < n; base += 64) {
@@ -545,6 +549,9 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
     const float my_key = mine < n ? s.dbuf[mine] : INFINITY;
     const uint32_t my_id = mine < n ? s.nbuf[mine] : 0u;
     unsigned long long todo = __ballot(mine < n && my_id != kEmpty && (st.top_size < ef || st.lower > my_key));
+    unsigned long long marked = 0ull;
+    if (NS == 0 && deleted != nullptr)
+      marked = __ballot(mine < n && my_id != kEmpty && ((deleted[my_id >> 5] >> (my_id & 31u)) & 1u) != 0u);
     while (todo != 0ull) {
       const int j = __builtin_ctzll(todo);
       todo &= todo - 1ull;
@@ -574,10 +581,13 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
             st.lower = st.n_acc >= ef ? topkeys_max<NS>(tk) : st.maxkey;  // hnswlib's lowerBound
           } else {
             LdsHeap top{s.top};
-            coop_push<false>(top, st.top_size, e, lane);
-            if (st.top_size > ef) coop_pop<false>(top, st.top_size, s.tree, lane);
+            if (((marked >> j) & 1ull) == 0ull) {
+              coop_push<false>(top, st.top_size, e, lane);
+              if (st.top_size > ef) coop_pop<false>(top, st.top_size, s.tree, lane);
+            }
             wave_sync();
-            st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
+            if (st.top_size > 0)
+              st.lower = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s.top[0].key)));
           }
         }
       }
@@ -590,10 +600,12 @@ __device__ __forceinline__ void accept_list(Scratch& s, SearchState& st, TopKeys
 // On entry s.nbuf[0..n_seed) holds seed ids that are already marked visited.  On exit
 // the accepted entries are in s.log[0..st.n_acc) and tk holds the result keys (NS > 0), or
 // s.top[0..st.top_size) is the literal result max-heap (NS == 0).  BUILD selects hnswlib's
-// construction-time stop rule.
+// construction-time stop rule; so do delete marks (see accept_list): a result heap short of ef never stops
+// the search, marked candidates beyond the bound are walked through.
 template <int DT, int QR, int NS, bool BUILD>
 __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>& qv, int level, int ef, Scratch& s,
-                                             SearchState& st, TopKeys<NS>& tk, int n_seed, int lane) {
+                                             SearchState& st, TopKeys<NS>& tk, int n_seed, int lane,
+                                             const uint32_t* deleted = nullptr) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int S = row_stride(ix, level);
   int n = n_seed;
@@ -604,11 +616,11 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
   while (true) {
     wave_sync();
     int cid = -1;
-    accept_list<NS>(s, st, tk, n, ef, lane);
+    accept_list<NS>(s, st, tk, n, ef, lane, deleted);
     if (!st.fail && st.cand_size > 0) {
       wave_sync();
       const HeapEnt c = uniform_ent(s.cand[0]);
-      const bool stop = BUILD ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
+      const bool stop = (BUILD || (NS == 0 && deleted != nullptr)) ? (c.key > st.lower && st.top_size == ef) : (c.key > st.lower);
       if (!stop) {
         cid = (int)c.id;
         if (st.cand_size <= s.cand_lds) {

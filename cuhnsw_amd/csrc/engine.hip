@@ -200,6 +200,7 @@ class Engine {
   int Dp = 0;
   DevBuf<float> d_vectors;
   DevBuf<uint64_t> d_labels;
+  DevBuf<uint32_t> d_deleted;  // one bit per element: hnswlib's delete marks of a loaded file (used while host.n_deleted > 0)
   DevBuf<uint32_t> d_links0, d_linksU;
   DevBuf<int64_t> d_upper_off;
   DevBuf<int> d_levels;
@@ -383,6 +384,8 @@ class Engine {
     host.layout_links();
     host.labelled = false;
     host.labels.clear();
+    host.deleted.clear();  // a graph built anew holds every element
+    host.n_deleted = 0;
     have_levels = true;
     have_graph = false;
     if (has_device) upload_structure();
@@ -862,10 +865,20 @@ class Engine {
     a.lcap = (std::max(std::max(host.S0, host.SU), std::max(k, 64)) + 63) / 64 * 64;
     const int q = qr();
     size_t fixed = (size_t)a.lcap * 8 + (q == 0 ? (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16 : 0);
-    const int ns = key_slots(ef);
+    int ns = key_slots(ef);
     a.vc_bits = auto_vc_bits();
     a.fast_path = no_alloc ? 2 : (fast_suspended ? 0 : fast_path);
     a.reverse = opt.reverse_cand ? 1 : 0;
+    // An index with deleted elements (hnswlib's marks in a loaded file) is searched by hnswlib's rule for them:
+    // walked through, never returned.  Only the search on the literal queues in LDS states that rule; it takes
+    // every query of such an index.
+    if (host.n_deleted > 0) {
+      if (no_alloc) throw std::runtime_error("search_knn (no allocation): the index holds deleted elements");
+      if (a.reverse) throw std::runtime_error("search_knn: reverse_cand is not defined on an index with deleted elements");
+      ns = 0;
+      a.fast_path = 0;
+      a.deleted = d_deleted.p;
+    }
     // reverse_cand: the sorted set in registers expands its farthest entry; beyond its capacity (ef >= 1024) the
     // literal pass does, on a sorted list in LDS
     if (a.reverse) a.fast_path = ns > 0 ? 2 : 0;
@@ -1152,6 +1165,14 @@ class Engine {
       upload_links();
       d_labels.reserve((size_t)host.N);
       HIP_CHECK(hipMemcpyAsync(d_labels.p, host.labels.data(), (size_t)host.N * 8, hipMemcpyHostToDevice, stream));
+      std::vector<uint32_t> marks;
+      if (host.n_deleted > 0) {
+        marks.assign(((size_t)host.N + 31) / 32, 0u);
+        for (int i = 0; i < host.N; ++i)
+          if (host.deleted[i]) marks[(size_t)i >> 5] |= 1u << (i & 31);
+        d_deleted.reserve(marks.size());
+        HIP_CHECK(hipMemcpyAsync(d_deleted.p, marks.data(), marks.size() * 4, hipMemcpyHostToDevice, stream));
+      }
       HIP_CHECK(hipStreamSynchronize(stream));
       pool_slots = 0;  // N may have changed: rebuild the slot pool lazily
       pool = SlotPool{};
@@ -1267,6 +1288,7 @@ int cuhnsw_max_level(cuhnsw_engine* e) { return e ? e->impl.host.maxlevel : 0; }
 int cuhnsw_enter_point(cuhnsw_engine* e) { return e ? (int)e->impl.host.enterpoint : 0; }
 int cuhnsw_has_device(void) { return cuhnsw_amd::device_present() ? 1 : 0; }
 double cuhnsw_last_build_seconds(cuhnsw_engine* e) { return e ? e->impl.last_build_seconds : 0.0; }
+int cuhnsw_num_deleted(cuhnsw_engine* e) { return e ? e->impl.host.n_deleted : 0; }
 int cuhnsw_last_search_repeats(cuhnsw_engine* e) { return e ? e->impl.last_repeats : 0; }
 int cuhnsw_last_search_trails(cuhnsw_engine* e) { return e ? e->impl.last_trails : 0; }
 int cuhnsw_last_search_side_by_side(cuhnsw_engine* e) { return e ? e->impl.last_side_by_side : 0; }

@@ -63,6 +63,8 @@ void wr(FILE* f, const void* p, size_t n) {
 void rd(FILE* f, void* p, size_t n, const char* what) {
   if (n && std::fread(p, 1, n, f) != n) throw std::runtime_error(std::string("index file: truncated ") + what);
 }
+constexpr uint32_t kDeleteMark = 0x00010000u;  // hnswlib's DELETE_MARK as a bit of the level-0 count word
+
 int row_degree(const uint32_t* row, int cap) {
   int d = 0;
   while (d < cap && row[d] != kEmpty) ++d;
@@ -103,8 +105,9 @@ void write_index_file(const HostIndex& ix, const std::string& path) {
     std::memset(rec.data(), 0, rec.size());  // unused link slots are written as zeros
     const uint32_t* row = &ix.links0[(size_t)i * ix.S0];
     uint32_t deg = (uint32_t)row_degree(row, ix.max_m0);
+    if (ix.n_deleted > 0 && ix.deleted[i]) deg |= kDeleteMark;
     std::memcpy(rec.data(), &deg, 4);
-    std::memcpy(rec.data() + 4, row, (size_t)deg * 4);
+    std::memcpy(rec.data() + 4, row, (size_t)(deg & 0xffffu) * 4);
     std::memcpy(rec.data() + h.offset_data, &ix.vectors[(size_t)i * ix.D], (size_t)ix.D * 4);
     uint64_t label = ix.labels.empty() ? (uint64_t)i : ix.labels[i];
     std::memcpy(rec.data() + h.label_offset, &label, 8);
@@ -158,6 +161,8 @@ void read_index_file(HostIndex& ix, const std::string& path) {
   ix.vectors.resize((size_t)ix.N * ix.D);
   ix.labels.resize(ix.N);
   ix.levels.assign(ix.N, 0);
+  ix.deleted.clear();
+  ix.n_deleted = 0;
   const int S0 = HostIndex::stride0(ix.max_m0);
   std::vector<uint32_t> l0((size_t)ix.N * S0, kEmpty);
   std::vector<unsigned char> rec(h.size_data_per_element);
@@ -166,13 +171,14 @@ void read_index_file(HostIndex& ix, const std::string& path) {
     uint32_t word;
     std::memcpy(&word, rec.data(), 4);
     uint32_t deg = word & 0xffffu;  // hnswlib keeps the count in the low 16 bits, flags above
-    // hnswlib's markDelete sets bit 0 of the word's third byte.  A deleted element is still walked through
-    // by hnswlib's search but never returned, which this engine's search does not reproduce: refuse the
-    // file rather than hand deleted elements back as results (the reference reads the word as a plain
-    // count, cpp/src/cuhnsw_base.cu:311-312, and would index out of its rows).
-    if (word & 0x00010000u)
-      throw std::runtime_error("index file: element " + std::to_string(i) +
-                               " is marked deleted (hnswlib markDelete); files with deleted elements are not supported");
+    // hnswlib's markDelete sets bit 0 of the word's third byte; the other flag bits are unknown and dropped
+    // (the reference reads the word as a plain count, cpp/src/cuhnsw_base.cu:311-312, and would index out
+    // of its rows)
+    if (word & kDeleteMark) {
+      if (ix.deleted.empty()) ix.deleted.assign(ix.N, 0);
+      ix.deleted[i] = 1;
+      ++ix.n_deleted;
+    }
     if (deg > (uint32_t)ix.max_m0) throw std::runtime_error("index file: link count above max_m0");
     uint32_t* row = &l0[(size_t)i * S0];
     std::memcpy(row, rec.data() + 4, (size_t)deg * 4);

@@ -27,6 +27,12 @@ struct HostIndex {
   std::vector<int64_t> upper_off;      // N: index of the node's level-1 row in linksU, -1 if none
   std::vector<uint32_t> linksU;        // (sum of levels) x SU; row of (node, level) = upper_off[node] + level - 1
   int64_t upper_rows = 0;
+  // hnswlib's delete marks (markDelete: bit 0 of the third byte of an element's level-0 count word), one
+  // byte per element, or empty when nothing is marked.  A marked element is searched through like any
+  // other and never returned.  The reference keeps no such mark: it reads the count word as a plain count
+  // (cpp/src/cuhnsw_base.cu:311-312).
+  std::vector<uint8_t> deleted;
+  int n_deleted = 0;
 
   static int stride0(int max_m0) { return (max_m0 + 31) / 32 * 32; }
   static int strideU(int max_m) { return (max_m + 15) / 16 * 16; }

@@ -68,6 +68,7 @@ struct SearchArgs {
   int fc_bits;  // log2 sets (two tags each) of the LDS visited filter of the sorted-set search, 0 = that search is off
   int fast_path;  // 0 = literal queues only (exact evaluation counters)
   int reverse;    // expand the farthest waiting candidate (reverse_cand); sorted-set pass only
+  const uint32_t* deleted;  // one bit per element (hnswlib's delete marks) or null; literal queues in LDS only (NS == 0)
   int lean;       // literal pass: result set = sorted set with ids, visited = LDS filter of 2^lean sets
                   // (no bitmap, evaluation counters include repeats); 0 = exact bitmap
   // Sorted-set pass with its queries taken longest first (entry_kernel and the two order kernels below); all
@@ -759,7 +760,7 @@ __global__ void __launch_bounds__(64, (QR >= 1 && QR <= 2 && NS > 0 && NS <= 5) 
     visit_single(s, st, cur, lane);
     if (lane == 0) s.nbuf[0] = cur;
     wave_sync();
-    search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane);
+    search_level<DT, QR, NS, false>(ix, qv, 0, a.ef, s, st, tk, 1, lane, NS == 0 ? a.deleted : nullptr);
 
     // the k best.  With the keys in registers: the entries of the log at or below the k-th
     // key are the answer unless equal keys straddle the cut; then (and for NS == 0) the

@@ -65,7 +65,14 @@ int cuhnsw_build_graph(cuhnsw_engine* e);
 int cuhnsw_save_index(cuhnsw_engine* e, const char* fpath);
 /* void CuHNSW::LoadIndex(std::string fpath) (cpp/src/cuhnsw_base.cu:250-365):
  * after it, search returns the file's labels instead of internal ids
- * (cpp/src/cuhnsw_build.cu:284-286). */
+ * (cpp/src/cuhnsw_build.cu:284-286).
+ * A file written by hnswlib may hold deleted elements (markDelete: bit 0 of the third byte of an element's
+ * level-0 count word; the reference reads that word as a plain count, cpp/src/cuhnsw_base.cu:311-312).  They
+ * are honoured the way hnswlib's search honours them: walked through, never returned (found_cnt may then be
+ * below topk), and cuhnsw_save_index writes the marks back.  Every query of such an index is answered by the
+ * search on the literal queues (several times slower than the usual two passes); reverse_cand and
+ * cuhnsw_search_knn_device_noalloc fail on it with a message.  cuhnsw_set_random_levels + cuhnsw_build_graph
+ * build a new graph over every element and drop the marks. */
 int cuhnsw_load_index(cuhnsw_engine* e, const char* fpath);
 
 /* void CuHNSW::SearchGraph(const float* qdata, int num_queries, int topk,
@@ -116,6 +123,8 @@ int cuhnsw_num_data(cuhnsw_engine* e);
 int cuhnsw_num_dims(cuhnsw_engine* e);
 int cuhnsw_max_level(cuhnsw_engine* e);
 int cuhnsw_enter_point(cuhnsw_engine* e);
+/* elements of the loaded index that carry hnswlib's delete mark (0 for an index built here) */
+int cuhnsw_num_deleted(cuhnsw_engine* e);
 /* 1 if a HIP device is usable by this process, else 0 */
 int cuhnsw_has_device(void);
 /* seconds spent inside the last cuhnsw_build_graph (device work, event-timed) */

@@ -44,6 +44,11 @@
 //                           (ef >= N); against the CUDA reference itself PARITY
 //                           UNPINNED: it cannot run here and leaves the order
 //                           among equal distances to its warp reduction.
+//   search_layer_deleted .. (hnswlib searchBaseLayerST on an index with deleted elements; the reference
+//                           has no such notion) pinned by brute force over the elements that are left
+//                           (ef >= N), by hand-walked chains whose only bridge is deleted and by
+//                           "no mark == the plain search" (tests/test_oracle_deleted.py); against a real
+//                           hnswlib binary PARITY UNPINNED.
 //   file format ........... pinned by closed-form byte layout fixtures
 //   select_reference ...... (the reference's SearchHeuristic incl. nn_num, save_remains, new_comer) pinned by
 //                           closed-form point sets, by a brute-force statement of HNSW Alg. 4 on integer
@@ -64,6 +69,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <limits>
 #include <mutex>
 #include <queue>
 #include <string>
@@ -134,9 +140,12 @@ struct Index {
   std::vector<uint32_t> links0;     // N x (1 + max_m0): count, ids
   std::vector<size_t> upper_off;    // N: offset (in uint32) into linksU, valid if levels[i] > 0
   std::vector<uint32_t> linksU;     // sum(levels) x (1 + max_m)
+  std::vector<uint8_t> deleted;     // N, or empty: hnswlib's delete marks (markDelete)
+  int n_deleted = 0;
   std::string error;
 
   const float* vec(uint32_t i) const { return &vectors[(size_t)i * D]; }
+  bool is_deleted(uint32_t i) const { return n_deleted > 0 && deleted[i] != 0; }
   uint32_t* list(uint32_t i, int level) {
     if (level == 0) return &links0[(size_t)i * (1 + max_m0)];
     return &linksU[upper_off[i] + (size_t)(level - 1) * (1 + max_m)];
@@ -192,6 +201,7 @@ static bool save_index(const Index& ix, const char* path) {
     std::memset(rec.data(), 0, rec.size());
     const uint32_t* l = ix.list(i, 0);
     std::memcpy(rec.data(), l, 4 + 4 * (size_t)l[0]);
+    if (ix.is_deleted((uint32_t)i)) rec[2] |= 0x01;  // hnswlib's DELETE_MARK: bit 0 of the count word's third byte
     std::memcpy(rec.data() + offsetData, ix.vec(i), (size_t)ix.D * 4);
     std::memcpy(rec.data() + label_offset, &ix.labels[i], 8);
     ok = std::fwrite(rec.data(), 1, rec.size(), f) == rec.size();
@@ -233,6 +243,8 @@ static bool load_index(Index& ix, const char* path) {
   ix.labels.resize(ix.N);
   ix.levels.assign(ix.N, 0);
   ix.links0.assign((size_t)ix.N * (1 + ix.max_m0), 0u);
+  ix.deleted.assign(ix.N, 0);
+  ix.n_deleted = 0;
   std::vector<char> rec(size_data_per_element);
   for (int i = 0; i < ix.N; ++i) {
     if (std::fread(rec.data(), 1, rec.size(), f) != rec.size()) { std::fclose(f); ix.error = "truncated level-0 block"; return false; }
@@ -241,6 +253,7 @@ static bool load_index(Index& ix, const char* path) {
     uint32_t cnt = word & 0xffffu;  // hnswlib keeps the count in the low 16 bits
     if (cnt > (uint32_t)ix.max_m0) { std::fclose(f); ix.error = "bad link count"; return false; }
     l[0] = cnt;
+    if (word & 0x00010000u) { ix.deleted[i] = 1; ix.n_deleted++; }  // (hnswlib counts its marks the same way on load)
     std::memcpy(l + 1, rec.data() + 4, 4 * (size_t)cnt);
     std::memcpy(&ix.vectors[(size_t)i * ix.D], rec.data() + offsetData, (size_t)ix.D * 4);
     std::memcpy(&ix.labels[i], rec.data() + label_offset, 8);
@@ -328,6 +341,52 @@ static MaxQueue search_layer(const Index& ix, const float* q, uint32_t ep, float
       if (top.size() < ef || lowerBound > d) {
         cand.emplace(-d, n);
         top.emplace(d, n);
+        if (top.size() > ef) top.pop();
+        if (!top.empty()) lowerBound = top.top().first;
+        if (c && (long long)cand.size() > c->max_cand) c->max_cand = (long long)cand.size();
+      }
+    }
+  }
+  return top;
+}
+
+// hnswlib searchBaseLayerST as it runs on an index that holds deleted elements (its has_deletions /
+// non-bare-bone form, no filter): a deleted element is visited, evaluated, queued and expanded like any
+// other, but never enters the result queue; the search stops only once the result queue is FULL and the
+// nearest candidate lies beyond its largest key (a queue still short of ef never stops it: deleted
+// candidates beyond the bound are walked through); the bound moves only while the result queue holds
+// something.  A deleted entry point is queued with the largest float as its key and is not evaluated by
+// hnswlib; it is the queue's only entry when it is taken, so its key decides nothing, and the evaluation
+// is counted here as for any entry point.  The reference itself knows no deleted elements (it reads the
+// count word as a plain count, cpp/src/cuhnsw_base.cu:311-312).
+static MaxQueue search_layer_deleted(const Index& ix, const float* q, uint32_t ep, float dep, int level, size_t ef,
+                                     Visited& vis, Counters* c) {
+  MaxQueue top, cand;
+  float lowerBound;
+  if (!ix.is_deleted(ep)) {
+    lowerBound = dep;
+    top.emplace(dep, ep);
+    cand.emplace(-dep, ep);
+  } else {
+    lowerBound = std::numeric_limits<float>::max();
+    cand.emplace(-lowerBound, ep);
+  }
+  vis.test_and_set(ep);
+  while (!cand.empty()) {
+    DistId cur = cand.top();
+    if ((-cur.first) > lowerBound && top.size() == ef) break;
+    cand.pop();
+    if (c) c->n_hops++;
+    const uint32_t* l = ix.list(cur.second, level);
+    uint32_t cnt = l[0];
+    for (uint32_t j = 0; j < cnt; ++j) {
+      uint32_t n = l[1 + j];
+      if (vis.test_and_set(n)) continue;
+      float d = canon_dist(q, ix.vec(n), ix.D, ix.dist_type);
+      if (c) c->n_dist++;
+      if (top.size() < ef || lowerBound > d) {
+        cand.emplace(-d, n);
+        if (!ix.is_deleted(n)) top.emplace(d, n);
         if (top.size() > ef) top.pop();
         if (!top.empty()) lowerBound = top.top().first;
         if (c && (long long)cand.size() > c->max_cand) c->max_cand = (long long)cand.size();
@@ -435,7 +494,9 @@ static int search_one(const Index& ix, const float* q, int k, int ef, Visited& v
   for (int level = ix.maxlevel; level > 0; --level) descend_level(ix, q, level, cur, dcur, c);
   vis.reset(ix.N);
   if (c) c->n_dist++;  // the entry's level-0 evaluation is counted once
-  MaxQueue top = search_layer(ix, q, cur, dcur, 0, (size_t)std::max(ef, k), vis, c);
+  // (hnswlib: the bare-bone search while nothing is marked deleted, the other form as soon as something is)
+  MaxQueue top = ix.n_deleted > 0 ? search_layer_deleted(ix, q, cur, dcur, 0, (size_t)std::max(ef, k), vis, c)
+                                  : search_layer(ix, q, cur, dcur, 0, (size_t)std::max(ef, k), vis, c);
   while ((int)top.size() > k) top.pop();
   std::vector<std::pair<float, uint64_t>> res;
   std::vector<uint32_t> internal;
@@ -689,6 +750,7 @@ int orc_from_arrays(void* h, const float* vectors, int N, int D, const int* leve
   if (!ix.linksU.empty()) std::memcpy(ix.linksU.data(), linksU, ix.linksU.size() * 4);
   ix.labels.resize(N);
   for (int i = 0; i < N; ++i) ix.labels[i] = labels ? labels[i] : (uint64_t)i;
+  ix.deleted.clear(); ix.n_deleted = 0;
   return 1;
 }
 
@@ -701,10 +763,24 @@ int orc_build(void* h, const float* data, int N, int D, const int* levels, int d
   ix.ef_construction = ef_construction; ix.mult = mult;
   ix.vectors.assign(data, data + (size_t)N * D);
   ix.levels.assign(levels, levels + N);
+  ix.deleted.clear(); ix.n_deleted = 0;
   build_index(ix, threads > 0 ? threads : 1);
   return 1;
 }
 
+// hnswlib markDelete / unmarkDelete on internal ids; returns the number of marked elements, -1 on a bad id
+int orc_mark_deleted(void* h, const unsigned* ids, int n, int mark) {
+  Index& ix = *static_cast<Index*>(h);
+  if ((int)ix.deleted.size() != ix.N) ix.deleted.assign(ix.N, 0);
+  for (int i = 0; i < n; ++i) {
+    if (ids[i] >= (unsigned)ix.N) return -1;
+    ix.deleted[ids[i]] = mark ? 1 : 0;
+  }
+  ix.n_deleted = 0;
+  for (int i = 0; i < ix.N; ++i) ix.n_deleted += ix.deleted[i] ? 1 : 0;
+  return ix.n_deleted;
+}
+int orc_num_deleted(void* h) { return static_cast<Index*>(h)->n_deleted; }
 int orc_num_data(void* h) { return static_cast<Index*>(h)->N; }
 int orc_num_dims(void* h) { return static_cast<Index*>(h)->D; }
 int orc_maxlevel(void* h) { return static_cast<Index*>(h)->maxlevel; }

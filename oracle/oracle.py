@@ -51,8 +51,9 @@ def lib():
         ctypes.c_void_p, _c_float_p, ctypes.c_int, ctypes.c_int, _c_int_p,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_double, ctypes.c_int]
+    l.orc_mark_deleted.argtypes = [ctypes.c_void_p, _c_uint_p, ctypes.c_int, ctypes.c_int]
     for name in ("orc_num_data", "orc_num_dims", "orc_maxlevel", "orc_max_m",
-                 "orc_max_m0", "orc_validate"):
+                 "orc_max_m0", "orc_validate", "orc_num_deleted"):
       getattr(l, name).argtypes = [ctypes.c_void_p]
     l.orc_enterpoint.argtypes = [ctypes.c_void_p]
     l.orc_enterpoint.restype = ctypes.c_uint
@@ -189,6 +190,16 @@ class OracleIndex:
   enterpoint = property(lambda s: s._l.orc_enterpoint(s._h))
   max_m = property(lambda s: s._l.orc_max_m(s._h))
   max_m0 = property(lambda s: s._l.orc_max_m0(s._h))
+  num_deleted = property(lambda s: s._l.orc_num_deleted(s._h))
+
+  def mark_deleted(self, ids, mark=True):
+    """hnswlib markDelete (unmarkDelete with mark=False) on internal ids; the marks are written by save()
+    and honoured by search(): walked through, never returned."""
+    ids = np.ascontiguousarray(ids, dtype=np.uint32).ravel()
+    n = self._l.orc_mark_deleted(self._h, _p(ids, _c_uint_p), ids.size, 1 if mark else 0)
+    if n < 0:
+      raise ValueError("mark_deleted: id out of range")
+    return n
 
   def levels(self):
     out = np.empty(self.num_data, dtype=np.int32)

@@ -408,7 +408,8 @@ def test_search_on_a_file_with_spare_capacity_and_flag_bits(oracle, tmp_path):
   """An index file as hnswlib writes it from an index that was not filled up (max_elements >
   cur_element_count: extra level-0 records of arbitrary content) and with unknown flag bits set above
   the 16-bit link counts: loaded on the GPU it must answer exactly as the oracle does on the compact
-  file; the same file with one element marked deleted is refused."""
+  file; so must the same file with elements marked deleted (hnswlib markDelete), against the oracle that
+  read the same marks."""
   import struct
   n, d = 4000, 20
   x = gauss_mixture(n, d, seed=31)
@@ -437,9 +438,103 @@ def test_search_on_a_file_with_spare_capacity_and_flag_bits(oracle, tmp_path):
   (word,) = struct.unpack_from("<I", marked, 96 + 5 * rec)
   struct.pack_into("<I", marked, 96 + 5 * rec, word | (1 << 16))   # hnswlib's markDelete on element 5
   open(p2, "wb").write(bytes(marked))
-  with pytest.raises(RuntimeError, match="marked deleted"):
-    e.load_index(p2)
-  _check_parity(oracle, ix, e, q[:20], 10, 80, counters=False)     # the refused load left the resident index alone
+  e.load_index(p2)
+  assert e.num_deleted == 1
+  ix.mark_deleted([5])
+  _check_deleted_parity(ix, e, q, 10, 80)
+
+
+def _check_deleted_parity(ix, e, q, k, ef):
+  """Engine against oracle on an index with deleted elements: ids, distances, found counts and every
+  counter (the search on the literal queues evaluates exactly what hnswlib's loop evaluates)."""
+  o_ids, o_d, o_f, o_cnt = ix.search(q, k, ef, counters=True)
+  g_ids, g_d, g_f, stats = _device_search(e, q, k, ef)
+  assert (g_f == o_f).all()
+  for r in range(q.shape[0]):
+    f = o_f[r]
+    assert (g_ids[r, :f] == o_ids[r, :f]).all(), "query %d" % r
+    assert (g_d[r, :f] == o_d[r, :f]).all()
+    assert (g_ids[r, f:] == -1).all()
+  assert (stats == o_cnt[:, :4]).all()
+  h_ids, h_d, h_f = e.search_knn(q, k, ef)
+  assert (h_ids == g_ids).all() and (h_f == g_f).all()
+
+
+@pytest.mark.parametrize("dist_type", ["dot", "l2"])
+def test_search_on_an_index_with_deleted_elements(oracle, tmp_path, dist_type):
+  """hnswlib's delete marks in a loaded file: walked through, never returned.  Shares from one element to
+  nearly all, the entry point among them, more results asked for than elements are left, the marks written
+  back by save_index; calls that cannot honour the marks fail with a message."""
+  n, d = 5000, 24
+  x = gauss_mixture(n, d, seed=41, normalise=(dist_type == "dot"))
+  q = gauss_mixture(200, d, seed=42, normalise=(dist_type == "dot"))
+  levels = _levels(n, 0.4, 43)
+  ix = oracle.OracleIndex(dist_type).build(x, levels, 8, 16, 60, 0.4)
+  rng = np.random.default_rng(44)
+  e = _engine(tmp_path, dist_type=dist_type, max_m=8, max_m0=16)
+  for share in (0.0002, 0.05, 0.5, 0.97, 0.999):
+    ix.mark_deleted(np.arange(n), mark=False)
+    dead = rng.choice(n, max(1, int(n * share)), replace=False)
+    dead = np.union1d(dead, [ix.enterpoint]) if share >= 0.05 else dead
+    ix.mark_deleted(dead)
+    p = str(tmp_path / ("m%g.idx" % share))
+    ix.save(p)
+    e.load_index(p)
+    assert e.num_deleted == dead.size
+    for k, ef in ((10, 64), (1, 1), (10, 300), (40, 20), (10, 1100)):
+      _check_deleted_parity(ix, e, q, k, ef)
+    ids, _, found = e.search_knn(q, 10, 64)
+    assert not np.isin(ids[ids >= 0], dead).any()
+    if share == 0.999:
+      assert (found == n - dead.size).all()     # five elements are left: every search finds them all
+    p2 = str(tmp_path / "back.idx")
+    e.save_index(p2)
+    assert open(p2, "rb").read() == open(p, "rb").read()
+  with pytest.raises(RuntimeError, match="deleted elements"):
+    e.search_knn_device_noalloc(0, 8, 10, 64, 0, 0, 0)   # (fails before any pointer is used)
+  # everything marked: nothing is found
+  ix.mark_deleted(np.arange(n))
+  p = str(tmp_path / "all.idx")
+  ix.save(p)
+  e.load_index(p)
+  ids, dist, found = e.search_knn(q[:50], 5, 40)
+  assert (found == 0).all() and (ids == -1).all()
+  # a graph built anew holds every element again
+  e.set_random_levels(levels)
+  e.build_graph()
+  assert e.num_deleted == 0
+  _, _, found = e.search_knn(q[:50], 5, 40)
+  assert (found == 5).all()
+
+
+def test_deleted_elements_and_equal_keys(oracle, tmp_path):
+  """Integer data: nearly every search meets equal keys, the order the literal heaps give them is the
+  answer; a third of the elements deleted."""
+  n, d = 6000, 8
+  x = integer_vectors(n, d, seed=51, hi=6)
+  q = integer_vectors(300, d, seed=52, hi=6)
+  levels = _levels(n, 0.4, 53)
+  ix = oracle.OracleIndex("l2").build(x, levels, 8, 16, 60, 0.4)
+  ix.mark_deleted(np.arange(1, n, 3))
+  p = str(tmp_path / "ties.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="l2", max_m=8, max_m0=16)
+  e.load_index(p)
+  for k, ef in ((10, 100), (1, 30), (50, 50), (10, 400)):
+    _check_deleted_parity(ix, e, q, k, ef)
+
+
+def test_reverse_cand_refuses_an_index_with_deleted_elements(oracle, tmp_path):
+  n, d = 1000, 8
+  x = gauss_mixture(n, d, seed=61)
+  ix = oracle.OracleIndex("dot").build(x, _levels(n, 0.4, 62), 8, 16, 40, 0.4)
+  ix.mark_deleted([3])
+  p = str(tmp_path / "r.idx")
+  ix.save(p)
+  e = _engine(tmp_path, dist_type="dot", max_m=8, max_m0=16, reverse_cand=True)
+  e.load_index(p)
+  with pytest.raises(RuntimeError, match="reverse_cand is not defined"):
+    e.search_knn(x[:4], 3, 20)
 
 
 def test_errors(tmp_path):

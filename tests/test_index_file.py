@@ -68,9 +68,8 @@ def test_library_reader_writer_bytes(tmp_path):
 
 def test_library_reads_hnswlib_count_word_flags(tmp_path):
   """hnswlib keeps the link count in the low 16 bits of the count word; the bits above are flags.
-  Unknown flag bits are masked off.  Bit 0 of the third byte is hnswlib's delete mark: a deleted
-  element must never come back as a search result, which this engine's search does not implement, so
-  such a file is refused with a message that says why."""
+  Unknown flag bits are masked off.  Bit 0 of the third byte is hnswlib's delete mark: it is kept (the
+  search walks through such an element and never returns it) and written back by save_index."""
   raw = bytearray(expected_bytes())
   struct.pack_into("<I", raw, 96, 2 | (1 << 17) | (1 << 31))
   p, q = str(tmp_path / "a.idx"), str(tmp_path / "b.idx")
@@ -82,11 +81,16 @@ def test_library_reads_hnswlib_count_word_flags(tmp_path):
   size_data = 3 * 4 + 4 + 2 * 4 + 8
   struct.pack_into("<I", raw, 96 + size_data, 2 | (1 << 16))     # node 1 marked deleted
   open(p, "wb").write(bytes(raw))
-  with pytest.raises(RuntimeError, match="element 1 is marked deleted"):
-    e.load_index(p)
-  assert e.num_data == 3                                          # the failed load left the engine as it was
+  assert e.num_deleted == 0
+  e.load_index(p)
+  assert e.num_data == 3 and e.num_deleted == 1
   e.save_index(q)
-  assert open(q, "rb").read() == expected_bytes()
+  marked = bytearray(expected_bytes())
+  struct.pack_into("<I", marked, 96 + size_data, 2 | (1 << 16))
+  assert open(q, "rb").read() == bytes(marked)                    # the mark is back, the unknown flags are not
+  open(p, "wb").write(expected_bytes())
+  e.load_index(p)
+  assert e.num_deleted == 0                                       # the marks belong to the file they came from
 
 
 def spare_capacity_bytes(spare=2):
