@@ -135,7 +135,7 @@ def exact_topk(torch, data_dev, sq_dev, queries_dev, k, dot):
   return np.concatenate(out)
 
 
-def other_workload_rows(torch, capi, datasets, orc, tmpdir, name, efs, n_check=1000, n_recall=1000, steps=3):
+def other_workload_rows(torch, capi, datasets, orc, tmpdir, name, efs, n_check=1000, n_recall=1000, steps=5):
   """One of the other benchmark configurations at its full size, compactly: build seconds, and per ef_search the
   search time of the whole batch (device pointers, HIP events on the engine's stream), QPS, recall, the
   distance-gather roofline fraction counted like the headline's (distinct evaluations of a literal-only pass

@@ -182,6 +182,15 @@ struct QVec {
   float4 q[QR > 0 ? QR : 1];
 };
 
+// Long rows (the query is read from LDS): 16 lanes own a row, so a lane fetches every 16th chunk of it,
+// kLongB of them per round.  The LDS copy of the query is zero-padded to whole rounds (kLongB * 16 chunks),
+// so that a round reads it without guards.
+constexpr int kLongB = 8;
+__host__ __device__ inline int query_lds_chunks(int Dp) {
+  const int chunk_rows = ((Dp >> 2) + 15) / 16;
+  return (chunk_rows + kLongB - 1) / kLongB * kLongB * 16;
+}
+
 // fills the query holder from a row of D floats (any alignment)
 template <int QR>
 __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const float* src, int D, int Dp, int lane) {
@@ -198,7 +207,7 @@ __device__ __forceinline__ void load_query(QVec<QR>& qv, float4* qlds, const flo
       qv.q[k] = t;
     }
   } else {
-    const int chunks = ((Dp >> 2) + 15) / 16 * 16;
+    const int chunks = query_lds_chunks(Dp);
     for (int c = lane; c < chunks; c += 64) {
       int i = 4 * c;
       float4 t;
@@ -249,44 +258,94 @@ __device__ __forceinline__ void dist_pass(const void* rows, uint32_t rowlen, uin
 }
 
 // long rows: 16 lanes still own one row (the summation order is tied to 16 lanes), so a lane
-// has rowlen/16 chunks to fetch; they are issued eight at a time to keep eight loads per lane
-// in flight, the query chunks come from LDS
-template <int DT, bool RAW, bool HALF>
-__device__ __forceinline__ void dist_long(const void* rows, int rowlen, int used, const float4* qlds, const uint32_t* ids,
-                                          int n, float* out, int g, int sub) {
+// has rowlen/16 chunks to fetch; they are issued B at a time for each of U groups of four rows, to keep
+// U * B loads per lane in flight; the query chunks come from LDS, one read for all U groups.  Rounds that
+// lie wholly inside the rows' data carry no guards; the last one re-reads chunk 0 for chunks past the end
+// and multiplies zeros there (the LDS copy of the query is zero-padded to whole rounds).
+template <int DT, bool RAW, bool HALF, int U, int B>
+__device__ __forceinline__ void dist_long_pass(const void* rows, int rowlen, int used, const float4* qlds, const uint32_t* ids,
+                                               int r, int n, float* out, int g, int sub) {
+  static_assert(B == kLongB, "the LDS copy of the query is padded to rounds of kLongB chunk rows");
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-  const int nk = (used + 15) >> 4;
-  constexpr int B = 8;
-  for (int r = 0; r < n; r += 4) {
-    const int idx = r + g;
+  const int nk = (used + 15) >> 4;  // chunk rows that hold data
+  const int nfull = used >> 4;      // chunk rows that hold nothing else
+  uint64_t first[U];
+  float ax[U], ay[U], az[U], aw[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int idx = r + 4 * u + g;
     const uint32_t id = ids[idx < n ? idx : n - 1];
-    const uint64_t first = (uint64_t)id * (uint32_t)rowlen;
-    float ax = 0.f, ay = 0.f, az = 0.f, aw = 0.f;
-    for (int k0 = 0; k0 < nk; k0 += B) {
-      float4 v[B];
+    first[u] = (uint64_t)id * (uint32_t)rowlen;
+    ax[u] = ay[u] = az[u] = aw[u] = 0.f;
+  }
+  int k0 = 0;
+  for (; k0 + B <= nfull; k0 += B) {
+    float4 v[U][B];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const uint64_t at = first[u] + (uint32_t)(sub + 16 * (k0 + b));
+        v[u][b] = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
+      }
+    }
+    // (the round's query chunks are read in one go, ahead of the arithmetic: read one by one each would be
+    // waited for in turn, which is what a lone wavefront's time goes to)
+    float4 qq[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) qq[b] = qlds[sub + 16 * (k0 + b)];
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc4<DT>(qq[b], v[u][b], ax[u], ay[u], az[u], aw[u]);
+    }
+  }
+  if (k0 < nk) {  // (k0 + B > nfull >= nk - 1: one more round reaches the end)
+    float4 v[U][B];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int b = 0; b < B; ++b) {
         const int c = sub + 16 * (k0 + b);
-        const uint64_t at = first + (c < used ? c : 0);  // unconditional load
+        const uint64_t at = first[u] + (uint32_t)(c < used ? c : 0);  // unconditional load (chunk 0 past the end)
         const float4 t = HALF ? load_chunk_f16(rows, at) : load_chunk_f32(rows, at);
-        v[b] = c < used ? t : zero;
-      }
-#pragma unroll
-      for (int b = 0; b < B; ++b) {
-        // chunks past the row end multiply zeros (the LDS copy is padded to a multiple of 16
-        // chunks, so only indices below that are read)
-        const float4 qq = (k0 + b < nk) ? qlds[sub + 16 * (k0 + b)] : zero;
-        acc4<DT>(qq, v[b], ax, ay, az, aw);
+        v[u][b] = c < used ? t : zero;
       }
     }
-    const float key = finish16<DT, RAW>(ax, ay, az, aw);
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const float4 qq = qlds[sub + 16 * (k0 + b)];  // zeros past the end
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc4<DT>(qq, v[u][b], ax[u], ay[u], az[u], aw[u]);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const float key = finish16<DT, RAW>(ax[u], ay[u], az[u], aw[u]);
+    const int idx = r + 4 * u + g;
     if (sub == 0 && idx < n) out[idx] = key;
-    __builtin_amdgcn_wave_barrier();  // (the lanes meet again here, not at the loop's end: see trail_mark)
+  }
+  __builtin_amdgcn_wave_barrier();  // (the lanes meet again here, not at the loop's end: see trail_mark)
+}
+// U = 2: eight rows at a time while more than four are left (twice the loads in flight, 64 more registers:
+// for the search of few queries at a time, where a wavefront waits for its own loads and arithmetic in turn)
+template <int DT, bool RAW, bool HALF, int U>
+__device__ __forceinline__ void dist_long(const void* rows, int rowlen, int used, const float4* qlds, const uint32_t* ids,
+                                          int n, float* out, int g, int sub) {
+  int r = 0;
+  while (r < n) {
+    if (U >= 2 && n - r > 4) {
+      dist_long_pass<DT, RAW, HALF, (U >= 2 ? 2 : 1), kLongB>(rows, rowlen, used, qlds, ids, r, n, out, g, sub);
+      r += 8;
+    } else {
+      dist_long_pass<DT, RAW, HALF, 1, kLongB>(rows, rowlen, used, qlds, ids, r, n, out, g, sub);
+      r += 4;
+    }
   }
 }
 
 // keys of ids[0..n) (LDS) against the query -> out[0..n) (LDS).  n is wavefront-uniform.
-template <int DT, int QR, bool RAW, bool HALF>
+template <int DT, int QR, bool RAW, bool HALF, int WIDE = 1>
 __device__ __forceinline__ void dist_list_t(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds, const uint32_t* ids,
                                             int n, float* out, int lane) {
   const int g = lane >> 4, sub = lane & 15;
@@ -311,15 +370,16 @@ __device__ __forceinline__ void dist_list_t(const DevIndex& ix, const QVec<QR>& 
       }
     }
   } else {
-    dist_long<DT, RAW, HALF>(rows, rowlen, used, qlds, ids, n, out, g, sub);
+    dist_long<DT, RAW, HALF, WIDE>(rows, rowlen, used, qlds, ids, n, out, g, sub);
   }
 }
 // (the element type of the stored vectors is a property of the index: one scalar branch per list)
-template <int DT, int QR, bool RAW>
+// WIDE (long rows only): groups of four rows in flight, see dist_long
+template <int DT, int QR, bool RAW, int WIDE = 1>
 __device__ __forceinline__ void dist_list(const DevIndex& ix, const QVec<QR>& qv, const float4* qlds,
                                           const uint32_t* ids, int n, float* out, int lane) {
-  if (uni(ix.half) != 0) dist_list_t<DT, QR, RAW, true>(ix, qv, qlds, ids, n, out, lane);
-  else dist_list_t<DT, QR, RAW, false>(ix, qv, qlds, ids, n, out, lane);
+  if (uni(ix.half) != 0) dist_list_t<DT, QR, RAW, true, WIDE>(ix, qv, qlds, ids, n, out, lane);
+  else dist_list_t<DT, QR, RAW, false, WIDE>(ix, qv, qlds, ids, n, out, lane);
 }
 
 __device__ __forceinline__ const uint32_t* link_row(const DevIndex& ix, uint32_t node, int level) {
@@ -1087,12 +1147,13 @@ __device__ __forceinline__ int tie_free_phase(const DevIndex& ix, const QVec<QR>
                                               SearchState& st, Frontier<NS>& fr, int& n, int& hop_cid, int& resume_at,
                                               unsigned long long& accepted, Trail& tr, const TieWatch& watch, int lane) {
   constexpr int N = NS > 0 ? NS : 1;
+  constexpr int kWide = (QR == 0 && !BUILD && NS <= 8) ? 2 : 1;  // (the search on long rows: dist_long)
   // (said to be wavefront-uniform, so that they sit in scalar registers through the loop)
   const int w0 = WATCH ? uni(watch.id0) : -1, w1 = WATCH ? uni(watch.id1) : -1;
   const int w2 = WATCH ? uni(watch.id2) : -1, w3 = WATCH ? uni(watch.id3) : -1;
   const float w_hi = WATCH ? uni(watch.hi) : -INFINITY;
   while (true) {
-    if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    if (n > 0) dist_list<DT, QR, false, kWide>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
     st.n_dist += n;
     wave_sync();
     // (unconditional LDS reads at a clamped index, then a select: no exec-mask branches)
@@ -1208,6 +1269,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
                                                   SearchState& st, Frontier<NS>& fr, int n_seed, int lane,
                                                   bool far = false, bool whole_set = false, Trail* trail = nullptr) {
   const int S = row_stride(ix, level);
+  constexpr int kWide = (QR == 0 && !BUILD && NS <= 8) ? 2 : 1;  // (the search on long rows: dist_long)
   int n = n_seed;
   const bool exact = !BUILD && !far;  // the outcome has to be hnswlib's
   Trail no_trail;
@@ -1260,7 +1322,7 @@ __device__ __forceinline__ int search_level_fast(const DevIndex& ix, const QVec<
     }
     while (true) {
       if (resume_at < 0) {
-        if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+        if (n > 0) dist_list<DT, QR, false, kWide>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
         st.n_dist += n;
         wave_sync();
       }

@@ -155,7 +155,7 @@ __host__ __device__ inline LdsPlan plan_lds(int qr, int Dp, int ef, int cand_lds
   LdsPlan p;
   size_t o = 0;
   p.qlds = o;
-  if (qr == 0) o += (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16;
+  if (qr == 0) o += (size_t)query_lds_chunks(Dp) * 16;
   p.top = o; o = align16(o + (size_t)(ef + 1) * 8);
   p.cand = o; o = align16(o + (size_t)cand_lds * 8);
   p.vcache = o; o = align16(o + (vc_bits > 0 ? ((size_t)2 << vc_bits) : 0));
@@ -192,7 +192,7 @@ __host__ __device__ inline FastLdsPlan plan_fast_lds(int qr, int Dp, int lcap, i
   FastLdsPlan p;
   size_t o = 0;
   p.qlds = o;
-  if (qr == 0) o += (size_t)(((Dp >> 2) + 15) / 16 * 16) * 16;
+  if (qr == 0) o += (size_t)query_lds_chunks(Dp) * 16;
   p.fcache = o; o = align16(o + ((size_t)4 << fc_bits));
   p.nbuf = o; o = align16(o + (size_t)lcap * 4);
   p.dbuf = o; o = align16(o + (size_t)lcap * 4);
@@ -849,7 +849,7 @@ __device__ __forceinline__ void load_node_query_t(QVec<QR>& qv, float4* qlds, co
       qv.q[k] = c < used ? t : zero;
     }
   } else {
-    const int chunks = (used + 15) / 16 * 16;
+    const int chunks = query_lds_chunks(ix.Dp);
     wave_sync();
     for (int c = lane; c < chunks; c += 64) {
       const uint64_t at = first + (c < used ? c : 0);
