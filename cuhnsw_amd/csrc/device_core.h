@@ -668,6 +668,7 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
                                              const uint32_t* deleted = nullptr) {
   SplitHeap cand{s.cand, s.cand_glob, s.cand_lds};
   const int S = row_stride(ix, level);
+  constexpr int kWide = (QR == 0 && !BUILD && NS <= 8) ? 2 : 1;  // (the search on long rows: dist_long)
   int n = n_seed;
   if (n > 0) {
     dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
@@ -699,13 +700,13 @@ __device__ __forceinline__ void search_level(const DevIndex& ix, const QVec<QR>&
       const VisitPending vp = visit_issue(row, S, s, lane);
       wave_sync();
       n = vp.n_ask;
-      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      if (n > 0) dist_list<DT, QR, false, kWide>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
       wave_sync();
       st.n_dist += visit_commit(vp, s, st, lane);
     } else {
       n = visit_row(row, S, s, st, lane);
       wave_sync();
-      if (n > 0) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+      if (n > 0) dist_list<DT, QR, false, kWide>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
       st.n_dist += n;
     }
   }
@@ -1492,7 +1493,7 @@ __device__ __forceinline__ void search_level_lean(const DevIndex& ix, const QVec
   bool own_stretch = false;  // between two markers: hops this pass makes itself
   if (trail_hops > 0) st.n_dist += trail_n_dist;  // the evaluations that pass made up to the trail's end count as performed
   while (true) {
-    if (n > 0 && !from_trail) dist_list<DT, QR, false>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
+    if (n > 0 && !from_trail) dist_list<DT, QR, false, (QR == 0 && NS <= 8) ? 2 : 1>(ix, qv, s.qlds, s.nbuf, n, s.dbuf, lane);
     st.n_dist += from_trail ? 0 : n;
     wave_sync();
     for (int base = 0; base < n; base += 64) {
