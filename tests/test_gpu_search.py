@@ -539,6 +539,35 @@ def test_reverse_cand_refuses_an_index_with_deleted_elements(oracle, tmp_path):
     e.search_knn(x[:4], 3, 20)
 
 
+def test_tiny_batches_on_long_rows(oracle, tmp_path):
+  """Vectors of more than 256 dimensions (the query in LDS): every batch takes the first pass, a single query
+  too, and a query handed over out of a batch of one is answered by the literal pass beside it.  Integer data:
+  nearly every query is handed over.  Dimensions that end inside a fetch round, on one, and just past one."""
+  for case, d in enumerate((300, 512, 1030)):
+    n = 2500
+    x = integer_vectors(n, d, seed=70 + case, hi=3)
+    q = integer_vectors(12, d, seed=80 + case, hi=3)
+    ix = oracle.OracleIndex("l2").build(x, _levels(n, 0.4, 90 + case), 8, 16, 60, 0.4)
+    p = str(tmp_path / ("long%d.idx" % d))
+    ix.save(p)
+    (tmp_path / ("e%d" % d)).mkdir()
+    e = _engine(tmp_path / ("e%d" % d), dist_type="l2", max_m=8, max_m0=16)
+    e.load_index(p)
+    handed = 0
+    for nq in (1, 2, 12):
+      for k, ef in ((10, 100), (1, 1), (5, 300)):
+        for start in (0, 3):
+          qq = q[start:start + nq]
+          o_ids, o_d, o_f, o_cnt = ix.search(qq, k, ef, counters=True)
+          g_ids, g_d, g_f, stats = _device_search(e, qq, k, ef)
+          assert (g_f == o_f).all()
+          for r in range(qq.shape[0]):
+            assert (g_ids[r, :o_f[r]] == o_ids[r, :o_f[r]]).all() and (g_d[r, :o_f[r]] == o_d[r, :o_f[r]]).all()
+          assert (stats[:, 1:] == o_cnt[:, 1:4]).all()
+          handed += e.last_search_repeats
+    assert handed > 0
+
+
 def test_errors(tmp_path):
   e = _engine(tmp_path)
   e.set_data(np.zeros((8, 4), np.float32))
